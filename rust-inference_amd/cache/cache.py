@@ -31,11 +31,13 @@ PAGE_SIZE = 32   # tokens per page, as in the reference (src/kvcache.rs:12)
 @dataclass(frozen=True)
 class KVNeed:
     """Keys and values of ``kv_heads`` heads of ``head_dim`` for every token, or for
-    the last ``window`` tokens only.  ``v_dim``: the size of a value head where it is not ``head_dim``."""
+    the last ``window`` tokens only.  ``v_dim``: the size of a value head where it is not ``head_dim``.
+    ``keep_first``: with a window, a sequence's first tokens that stay however far the window has moved on."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
     v_dim: Optional[int] = None
+    keep_first: Optional[int] = None
 
     @property
     def value_dim(self) -> int:
@@ -63,7 +65,7 @@ class KVGroup:
     def __init__(self, need: KVNeed, entries: list[int], num_pages: int, num_slots: int,
                  max_pages_per_slot: int, page_size: int, dtype, device, allocate: bool):
         self.need, self.entries, self.page_size = need, list(entries), page_size
-        self.pool = PagePool(num_pages, page_size, num_slots, max_pages_per_slot, need.window)
+        self.pool = PagePool(num_pages, page_size, num_slots, max_pages_per_slot, need.window, need.keep_first)
         self.index_of = {e: i for i, e in enumerate(self.entries)}
         k_shape = (len(self.entries), num_pages, need.kv_heads, page_size, need.head_dim)
         v_shape = (len(self.entries), num_pages, need.kv_heads, need.value_dim, page_size)

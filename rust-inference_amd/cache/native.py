@@ -16,6 +16,7 @@ _SIGNATURES = {
     "ri_pool_pages_needed": ([c_void_p, c_int, c_long, c_long], c_int),
     "ri_pool_reserve": ([c_void_p, c_int, c_long, c_long], c_int),
     "ri_pool_trim": ([c_void_p, c_int, c_long], c_int),
+    "ri_pool_keep_first": ([c_void_p, c_int], c_int),
     "ri_pool_release": ([c_void_p, c_int], c_int),
     "ri_pool_check": ([c_void_p], c_int),
     "ri_cache_new": ([POINTER(c_void_p), c_int, c_int, c_int], c_void_p),

@@ -19,7 +19,7 @@ UNMAPPED = -1
 
 class PagePool:
     def __init__(self, num_pages: int, page_size: int, num_slots: int, max_pages_per_slot: int,
-                 window: int | None = None):
+                 window: int | None = None, keep_first: int | None = None):
         if page_size < 1 or num_pages < 1 or max_pages_per_slot < 1 or num_slots < 1:
             raise CacheError("page pool sizes must be positive")
         self.num_pages, self.page_size = num_pages, page_size
@@ -28,6 +28,9 @@ class PagePool:
         self.handle = self._lib.ri_pool_new(num_pages, page_size, num_slots, max_pages_per_slot, int(window or 0))
         if not self.handle:
             raise native.fail()
+        self.keep_first = int(keep_first or 0)          # a sequence's first tokens, which a window never drops
+        if self.keep_first:
+            native.check(self._lib.ri_pool_keep_first(self.handle, self.keep_first))
         # slot -> its pages by logical number, -1 where none is mapped: the pool's own memory
         self.tables = np.ctypeslib.as_array(self._lib.ri_pool_tables(self.handle), shape=(num_slots, max_pages_per_slot))
 

@@ -2,8 +2,9 @@ from .base import ModelConfig, read_config_json
 from .qwen3 import Qwen3Config
 from .zidepel import ZidepelConfig
 from .pisulorn import PisulornConfig
+from .zakelorn import ZakelornConfig
 from .registry import (Architecture, config_from_dict, known_architectures, load_config,
                        register_architecture, resolve_architecture)
 
-__all__ = ["ModelConfig", "Qwen3Config", "ZidepelConfig", "PisulornConfig", "Architecture", "read_config_json", "config_from_dict",
+__all__ = ["ModelConfig", "Qwen3Config", "ZidepelConfig", "PisulornConfig", "ZakelornConfig", "Architecture", "read_config_json", "config_from_dict",
            "known_architectures", "load_config", "register_architecture", "resolve_architecture"]

@@ -335,6 +335,8 @@ int ri_pool_free_count(void* pool);
 int ri_pool_pages_needed(void* pool, int slot, long length_before, long new_tokens);                  // the count
 int ri_pool_reserve(void* pool, int slot, long length_before, long new_tokens);
 int ri_pool_trim(void* pool, int slot, long length);
+// The first `tokens` positions of every sequence stay mapped however far a window has moved on.
+int ri_pool_keep_first(void* pool, int tokens);
 int ri_pool_release(void* pool, int slot);
 int ri_pool_check(void* pool);
 // Slots, every slot's length, and the pools (not owned) that the slots hold pages in.

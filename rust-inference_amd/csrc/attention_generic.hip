@@ -5,7 +5,9 @@
 //
 // score_j = (q . k_j) * scale, then, with a cap c > 0, score_j <- c tanh(score_j / c), then, with a slope per
 // query head, score_j <- score_j - slope_h (p - j); the query at position p
-// sees keys lo..p with lo = 0 or p - window + 1;
+// sees keys lo..p with lo = 0 or p - window + 1, and with keep_first > 0 also the keys 0..keep_first-1 that lie
+// before lo (the first tokens of a sequence stay visible behind the window); with a sink per query head the
+// softmax's denominator also holds exp(sink_h), which has no key and no value;
 // online softmax with running maximum m, running sum l and factor exp(m_old - m_new)
 // (the reference: src/attention.rs:117-149; its GPU form src/cuda/kernels.cu:345-405).
 //
@@ -48,7 +50,8 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
                          const TC* __restrict__ v_pages, const int32_t* __restrict__ tok_pos,
                          const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ page_table, int table_width,
                          int heads, int kv_heads, int head_dim, int v_dim, int page_size, int window, float scale,
-                         float softcap, const float* __restrict__ slopes) {
+                         float softcap, const float* __restrict__ slopes, int keep_first,
+                         const float* __restrict__ sinks) {
     extern __shared__ float qs[];                 // head_dim floats: the query
     __shared__ float ps[ATT_TILE];                // this tile's weights
     __shared__ long rowoff[ATT_TILE];             // element offset of each key's column in the value pool
@@ -65,9 +68,12 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
     __syncthreads();
 
     float m = -INFINITY, l = 0.f, acc = 0.f, acc2 = 0.f;      // channels tid and tid + 256
-    for (int tile = lo / ATT_TILE; tile <= qpos / ATT_TILE; ++tile) {
+    const int kept = min(keep_first, lo);         // keys 0..kept-1 are seen although they lie behind the window
+    const int lo_tile = lo / ATT_TILE, kept_tiles = (kept + ATT_TILE - 1) / ATT_TILE;
+    for (int tile = 0; tile <= qpos / ATT_TILE; ++tile) {
+        if (tile >= kept_tiles && tile < lo_tile) { tile = lo_tile - 1; continue; }      // (the same for the whole workgroup)
         const int j = tile * ATT_TILE + tid;
-        const bool valid = j >= lo && j <= qpos;
+        const bool valid = (j >= lo || j < kept) && j <= qpos;
         float s = -INFINITY;
         if (valid) {
             const long page_head = ((long)table[j / page_size] * kv_heads + kvh) * page_size;
@@ -99,16 +105,18 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
         if (tid < v_dim) {
             acc *= corr;
             acc2 *= corr;
-            const int first = max(lo, tile * ATT_TILE) - tile * ATT_TILE;
-            const int last = min(qpos, tile * ATT_TILE + ATT_TILE - 1) - tile * ATT_TILE;
+            const int base = tile * ATT_TILE;
+            const int last = min(qpos, base + ATT_TILE - 1) - base;
             const bool second = tid + ATT_TILE < v_dim;
-            for (int jj = first; jj <= last; ++jj) {
+            for (int jj = 0; jj <= last; ++jj) {
+                if (base + jj < lo && base + jj >= kept) continue;         // not seen: no weight, and no offset either
                 acc += ps[jj] * to_f32(v_pages[rowoff[jj] + (long)tid * page_size]);
                 if (second) acc2 += ps[jj] * to_f32(v_pages[rowoff[jj] + (long)(tid + ATT_TILE) * page_size]);
             }
         }
         __syncthreads();                                   // before the next tile overwrites ps and rowoff
     }
+    if (sinks) l += expf(sinks[h] - m);                    // the sink: a term of the denominator alone
     if (tid < v_dim) from_f32(out + ((size_t)t * heads + h) * v_dim + tid, acc / l);
     if (tid + ATT_TILE < v_dim) from_f32(out + ((size_t)t * heads + h) * v_dim + tid + ATT_TILE, acc2 / l);
 }
@@ -117,17 +125,19 @@ template <typename T, bool VEC>
 static void launch_attention(void* out, const void* q, int q_stride, const void* k_pages, const void* v_pages,
                              const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
                              int table_width, int tokens, int heads, int kv_heads, int head_dim, int v_dim,
-                             int page_size, int window, float scale, float softcap, const float* slopes, hipStream_t s) {
+                             int page_size, int window, float scale, float softcap, const float* slopes, int keep_first,
+                             const float* sinks, hipStream_t s) {
     attention_generic_kernel<T, T, VEC><<<dim3(tokens, heads), ATT_TILE, (size_t)head_dim * sizeof(float), s>>>(
         (T*)out, (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, tok_pos, tok_seq, page_table,
-        table_width, heads, kv_heads, head_dim, v_dim, page_size, window, scale, softcap, slopes);
+        table_width, heads, kv_heads, head_dim, v_dim, page_size, window, scale, softcap, slopes, keep_first, sinks);
 }
 
-extern "C" int ri_attention(void* out, const void* q, int act_dtype, int q_stride, const void* k_pages,
+extern "C" int ri_attention_kept(void* out, const void* q, int act_dtype, int q_stride, const void* k_pages,
                             const void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq,
                             const int32_t* page_table, int table_width, int tokens, int heads, int kv_heads,
                             int head_dim, int v_dim, int page_size, int window, float scale, float softcap,
-                            const float* slopes, void* stream) {
+                            const float* slopes, int keep_first, const float* sinks, void* stream) {
+    RI_REQUIRE(keep_first >= 0, "attention: %d first tokens kept", keep_first);
     RI_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                "attention: tokens %d, heads %d, kv heads %d", tokens, heads, kv_heads);
     RI_REQUIRE(head_dim >= 1 && head_dim <= ATT_MAX_HEAD_DIM, "attention: head_dim %d must be between 1 and %d", head_dim,
@@ -145,10 +155,20 @@ extern "C" int ri_attention(void* out, const void* q, int act_dtype, int q_strid
     const bool vec = head_dim % (act_dtype == RI_F32 ? 4 : 8) == 0 && (uintptr_t)k_pages % 16 == 0;
 #define RI_ATT_GO(T, V) launch_attention<T, V>(out, q, q_stride, k_pages, v_pages, tok_pos, tok_seq, page_table, \
                                                table_width, tokens, heads, kv_heads, head_dim, v_dim, page_size, window, scale, \
-                                               softcap, slopes, s)
+                                               softcap, slopes, window > 0 ? keep_first : 0, sinks, s)
     if (act_dtype == RI_F32) { if (vec) RI_ATT_GO(float, true); else RI_ATT_GO(float, false); }
     else                     { if (vec) RI_ATT_GO(bf16_t, true); else RI_ATT_GO(bf16_t, false); }
 #undef RI_ATT_GO
     RI_LAUNCH_CHECK("attention");
     return 0;
+}
+
+extern "C" int ri_attention(void* out, const void* q, int act_dtype, int q_stride, const void* k_pages,
+                            const void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq,
+                            const int32_t* page_table, int table_width, int tokens, int heads, int kv_heads,
+                            int head_dim, int v_dim, int page_size, int window, float scale, float softcap,
+                            const float* slopes, void* stream) {
+    return ri_attention_kept(out, q, act_dtype, q_stride, k_pages, v_pages, cache_dtype, tok_pos, tok_seq, page_table,
+                             table_width, tokens, heads, kv_heads, head_dim, v_dim, page_size, window, scale, softcap,
+                             slopes, 0, nullptr, stream);
 }

@@ -10,52 +10,127 @@
 
 #define EXPERTS_MAX 1024
 
-// One thread a token.
+// One wavefront a token.  The router's outputs are `outs` = experts + identity experts (an identity expert hands the
+// token's own row on, times its weight; it has no matrices and is the business of whoever adds the experts up).
+//   scores:  s = sigmoid(z) or softmax(z) over all outputs (float32; the softmax with its maximum taken off);
+//   choice:  by s + correction; with groups, the outputs form `groups` equal runs of neighbours, a group's score is
+//            its largest choice score, and only outputs of the `keep` best groups can be chosen (the others count as
+//            minus infinity); the `top` largest, the lower index on a tie;
+//   weights: the chosen outputs' s, divided by their sum (+ 1e-20) when `normalize`.
+// z rows have z_stride >= outs columns; with `extra`, extra[t, 0] is the sum of the weights of the identity experts
+// chosen and extra[t, 1] = sigmoid(z[t, outs]), the gate of an expert that every token uses, whose logit rides as one
+// more row of the router's matrix.
+#define ROUTE_SIGMOID 0
+#define ROUTE_SOFTMAX 1
 __global__ void __launch_bounds__(64)
 experts_route_kernel(int32_t* __restrict__ ids, float* __restrict__ weights, float* __restrict__ dense,
-                     const float* __restrict__ z, const float* __restrict__ correction, int tokens, int experts, int top) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= tokens) return;
-    const float* zt = z + (size_t)t * experts;
-    float* dt = dense + (size_t)t * experts;
-    for (int e = 0; e < experts; ++e) dt[e] = 0.f;
-    float sum = 0.f;
+                     float* __restrict__ extra, const float* __restrict__ z, int z_stride,
+                     const float* __restrict__ correction, int outs, int experts, int top, int kind, int normalize,
+                     int groups, int keep) {
+    __shared__ float sc[EXPERTS_MAX], ch[EXPERTS_MAX], gbest[EXPERTS_MAX];
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* zt = z + (size_t)t * z_stride;
+    float* dt = dense + (size_t)t * outs;
+    if (kind == ROUTE_SOFTMAX) {
+        float m = -INFINITY;
+        for (int e = lane; e < outs; e += RI_WAVE) m = fmaxf(m, zt[e]);
+        m = wave_max(m);
+        float sum = 0.f;
+        for (int e = lane; e < outs; e += RI_WAVE) {
+            const float v = expf(zt[e] - m);
+            sc[e] = v;
+            sum += v;
+        }
+        sum = wave_sum(sum);
+        for (int e = lane; e < outs; e += RI_WAVE) sc[e] = sc[e] / sum;
+    } else {
+        for (int e = lane; e < outs; e += RI_WAVE) sc[e] = 1.f / (1.f + expf(-zt[e]));
+    }
+    for (int e = lane; e < outs; e += RI_WAVE) {
+        ch[e] = sc[e] + correction[e];
+        dt[e] = 0.f;
+    }
+    __syncthreads();
+    if (groups > 1 && keep < groups) {
+        const int per = outs / groups;
+        for (int g = lane; g < groups; g += RI_WAVE) {
+            float best = -INFINITY;
+            for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, ch[e]);
+            gbest[g] = best;
+        }
+        __syncthreads();
+        for (int g = lane; g < groups; g += RI_WAVE) {
+            int ahead = 0;                                    // groups that come before this one: better, or as good and earlier
+            for (int o = 0; o < groups; ++o) ahead += gbest[o] > gbest[g] || (gbest[o] == gbest[g] && o < g);
+            if (ahead >= keep)
+                for (int e = g * per; e < (g + 1) * per; ++e) ch[e] = -INFINITY;
+        }
+        __syncthreads();
+    }
+    float sum = 0.f, identity = 0.f;
     for (int k = 0; k < top; ++k) {
         int best = -1;
-        float best_choice = 0.f, best_s = 0.f;
-        for (int e = 0; e < experts; ++e) {
-            if (dt[e] != 0.f) continue;                       // chosen already (marked below)
-            const float s = 1.f / (1.f + expf(-zt[e]));
-            const float c = s + correction[e];
-            if (best < 0 || c > best_choice) { best = e; best_choice = c; best_s = s; }
+        float best_choice = 0.f;
+        for (int e = lane; e < outs; e += RI_WAVE) {
+            const float c = ch[e];
+            if (c == -INFINITY && best >= 0) continue;
+            if (best < 0 || c > best_choice) { best = e; best_choice = c; }
         }
-        ids[(size_t)t * top + k] = best;
-        weights[(size_t)t * top + k] = best_s;
-        dt[best] = -1.f;                                      // a mark that no weight can be
-        sum += best_s;
+        // the wavefront's best: the larger choice score, the lower index on a tie; lanes without an output lose
+        for (int m = RI_WAVE / 2; m > 0; m >>= 1) {
+            const int ob = __shfl_xor(best, m, RI_WAVE);
+            const float oc = __shfl_xor(best_choice, m, RI_WAVE);
+            if (ob >= 0 && (best < 0 || oc > best_choice || (oc == best_choice && ob < best))) { best = ob; best_choice = oc; }
+        }
+        const float w = sc[best];
+        __syncthreads();
+        if (lane == 0) {
+            ids[(size_t)t * top + k] = best;
+            weights[(size_t)t * top + k] = w;
+            ch[best] = -INFINITY;
+        }
+        __syncthreads();
+        sum += w;
     }
-    const float inv = 1.f / (sum + 1e-20f);
-    for (int k = 0; k < top; ++k) {
-        const float w = weights[(size_t)t * top + k] * inv;
-        weights[(size_t)t * top + k] = w;
-        dt[ids[(size_t)t * top + k]] = w;
+    const float inv = normalize ? 1.f / (sum + 1e-20f) : 1.f;
+    if (lane == 0) {
+        for (int k = 0; k < top; ++k) {
+            const float w = weights[(size_t)t * top + k] * inv;
+            const int e = ids[(size_t)t * top + k];
+            weights[(size_t)t * top + k] = w;
+            dt[e] = w;
+            if (e >= experts) identity += w;
+        }
+        if (extra) {
+            extra[(size_t)t * 2] = identity;
+            extra[(size_t)t * 2 + 1] = z_stride > outs ? 1.f / (1.f + expf(-zt[outs])) : 0.f;
+        }
     }
+}
+
+// An expert's activation from its gate and up branches.  limit > 0: g = min(gate, limit), u = clamp(up, -limit,
+// limit), g sigmoid(1.702 g) (u + 1).  limit <= 0: the plain gated form silu(gate) * up.
+__device__ __forceinline__ float expert_act(float gate, float up, float limit) {
+    if (limit > 0.f) {
+        const float a = fminf(gate, limit);
+        const float u = fminf(fmaxf(up, -limit), limit);
+        return a / (1.f + expf(-1.702f * a)) * (u + 1.f);
+    }
+    return gate / (1.f + expf(-gate)) * up;
 }
 
 template <typename T>
 __global__ void __launch_bounds__(256)
-experts_activate_kernel(T* __restrict__ out, const T* __restrict__ gu, const float* __restrict__ dense, int experts, int ff,
-                        float limit) {
+experts_activate_kernel(T* __restrict__ out, const T* __restrict__ gu, const float* __restrict__ dense, int dense_stride,
+                        int experts, int ff, float limit) {
     const int t = blockIdx.x, e = blockIdx.y;
-    const float w = dense ? dense[(size_t)t * experts + e] : 1.f;        // no weights: every row is of its expert
+    const float w = dense ? dense[(size_t)t * dense_stride + e] : 1.f;   // no weights: every row is of its expert
     T* o = out + ((size_t)t * experts + e) * ff;
     const T* g = gu + ((size_t)t * experts + e) * 2 * ff;
     for (int i = threadIdx.x; i < ff; i += blockDim.x) {
         float v = 0.f;
         if (w != 0.f) {
-            const float a = fminf(to_f32(g[i]), limit);
-            const float u = fminf(fmaxf(to_f32(g[ff + i]), -limit), limit);
-            v = w * (a / (1.f + expf(-1.702f * a)) * (u + 1.f));
+            v = w * expert_act(to_f32(g[i]), to_f32(g[ff + i]), limit);
         }
         from_f32(o + i, v);
     }
@@ -68,10 +143,11 @@ experts_activate_kernel(T* __restrict__ out, const T* __restrict__ gu, const flo
 __global__ void __launch_bounds__(256)
 experts_gate_up_rows_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ x, const bf16_t* __restrict__ gu,
                             const int32_t* __restrict__ ids, const float* __restrict__ weights, int top, int ff, int dim,
-                            float limit) {
+                            float limit, int experts) {
     const int lane = threadIdx.x & 63, i = blockIdx.x * 4 + (threadIdx.x >> 6), pair = blockIdx.y;
     if (i >= ff) return;                                      // (whole wavefronts)
     const int e = ids[pair];
+    if (e >= experts) return;                                 // an identity expert has no rows: the sum below adds the token's own
     const bf16_t* xr = x + (size_t)(pair / top) * dim;
     const bf16_t* gr = gu + ((size_t)e * 2 * ff + i) * dim;
     const bf16_t* ur = gr + (size_t)ff * dim;
@@ -90,9 +166,8 @@ experts_gate_up_rows_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__
     u = wave_sum(u);
     if (lane == 0) {
         // the products' results pass through bfloat16, as they do where the products are kernels of their own
-        const float gg = fminf(bf16_to_f32(f32_to_bf16(g)), limit);
-        const float uu = fminf(fmaxf(bf16_to_f32(f32_to_bf16(u)), -limit), limit);
-        act[(size_t)pair * ff + i] = f32_to_bf16(weights[pair] * (gg / (1.f + expf(-1.702f * gg)) * (uu + 1.f)));
+        act[(size_t)pair * ff + i] = f32_to_bf16(weights[pair] * expert_act(bf16_to_f32(f32_to_bf16(g)),
+                                                                             bf16_to_f32(f32_to_bf16(u)), limit));
     }
 }
 
@@ -101,12 +176,17 @@ experts_gate_up_rows_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__
 // along a row); out: float32 [tokens, dim].
 __global__ void __launch_bounds__(256)
 experts_down_rows_kernel(float* __restrict__ out, const bf16_t* __restrict__ act, const bf16_t* __restrict__ down,
-                         const int32_t* __restrict__ ids, int top, int ff, int dim, int experts) {
+                         const int32_t* __restrict__ ids, int top, int ff, int dim, int experts,
+                         const bf16_t* __restrict__ x, const float* __restrict__ weights) {
     const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6), t = blockIdx.y;
     if (n >= dim) return;
-    float acc = 0.f;
+    float acc = 0.f, own = 0.f;
     for (int k = 0; k < top; ++k) {
         const int pair = t * top + k;
+        if (ids[pair] >= experts) {                           // an identity expert: the token's own row times the weight
+            own += weights[pair] * bf16_to_f32(x[(size_t)t * dim + n]);
+            continue;
+        }
         const bf16_t* wr = down + (size_t)n * experts * ff + (size_t)ids[pair] * ff;
         const bf16_t* ar = act + (size_t)pair * ff;
         for (int c = lane * 8; c < ff; c += 512) {
@@ -119,22 +199,21 @@ experts_down_rows_kernel(float* __restrict__ out, const bf16_t* __restrict__ act
         }
     }
     acc = wave_sum(acc);
-    if (lane == 0) out[(size_t)t * dim + n] = acc;
+    if (lane == 0) out[(size_t)t * dim + n] = acc + own;
 }
 
 extern "C" int ri_experts_few_tokens(float* out, void* act, const void* x, const void* gu, const void* down,
                                      const int32_t* ids, const float* weights, int tokens, int experts, int top, int ff,
                                      int dim, float limit, void* stream) {
-    RI_REQUIRE(tokens > 0 && experts >= 1 && top >= 1 && top <= experts, "experts_few_tokens: %d tokens, %d of %d experts",
-               tokens, top, experts);
+    RI_REQUIRE(tokens > 0 && experts >= 1 && top >= 1, "experts_few_tokens: %d tokens, %d of %d experts", tokens, top, experts);
     RI_REQUIRE(ff >= 8 && ff % 8 == 0 && dim >= 8 && dim % 8 == 0, "experts_few_tokens: sizes %d and %d must be multiples of 8", ff, dim);
     RI_REQUIRE((long)tokens * top <= 65535 && tokens <= 65535, "experts_few_tokens: %d tokens exceed one launch", tokens);
     hipStream_t s = (hipStream_t)stream;
     experts_gate_up_rows_kernel<<<dim3((ff + 3) / 4, tokens * top), 256, 0, s>>>(
-        (bf16_t*)act, (const bf16_t*)x, (const bf16_t*)gu, ids, weights, top, ff, dim, limit);
+        (bf16_t*)act, (const bf16_t*)x, (const bf16_t*)gu, ids, weights, top, ff, dim, limit, experts);
     RI_LAUNCH_CHECK("experts_few_tokens (gate and up)");
     experts_down_rows_kernel<<<dim3((dim + 3) / 4, tokens), 256, 0, s>>>(out, (const bf16_t*)act, (const bf16_t*)down, ids,
-                                                                       top, ff, dim, experts);
+                                                                       top, ff, dim, experts, (const bf16_t*)x, weights);
     RI_LAUNCH_CHECK("experts_few_tokens (down)");
     return 0;
 }
@@ -258,27 +337,86 @@ extern "C" int ri_experts_combine(float* out, const void* y, const int32_t* dest
     return 0;
 }
 
-extern "C" int ri_experts_route(int32_t* ids, float* weights, float* dense, const float* z, const float* correction,
-                                int tokens, int experts, int top, void* stream) {
-    RI_REQUIRE(tokens > 0 && experts >= 1 && experts <= EXPERTS_MAX && top >= 1 && top <= experts,
-               "experts_route: %d tokens, the %d best of %d experts (at most %d)", tokens, top, experts, EXPERTS_MAX);
-    experts_route_kernel<<<(tokens + 63) / 64, 64, 0, (hipStream_t)stream>>>(ids, weights, dense, z, correction, tokens,
-                                                                             experts, top);
+extern "C" int ri_experts_route_general(int32_t* ids, float* weights, float* dense, float* extra, const float* z, int z_stride,
+                                        const float* correction, int tokens, int outs, int experts, int top, int kind,
+                                        int normalize, int groups, int keep, void* stream) {
+    RI_REQUIRE(tokens > 0 && experts >= 0 && experts <= outs && outs >= 1 && outs <= EXPERTS_MAX && top >= 1 && top <= outs,
+               "experts_route: %d tokens, the %d best of %d outputs (%d experts; at most %d)", tokens, top, outs, experts, EXPERTS_MAX);
+    RI_REQUIRE(kind == ROUTE_SIGMOID || kind == ROUTE_SOFTMAX, "experts_route: score kind %d", kind);
+    RI_REQUIRE(groups >= 1 && outs % groups == 0 && keep >= 1 && keep <= groups && (long)keep * (outs / groups) >= top,
+               "experts_route: %d outputs in %d groups of which %d stay, for the %d best", outs, groups, keep, top);
+    RI_REQUIRE(z_stride >= outs, "experts_route: logit rows of %d for %d outputs", z_stride, outs);
+    experts_route_kernel<<<tokens, 64, 0, (hipStream_t)stream>>>(ids, weights, dense, extra, z, z_stride, correction, outs,
+                                                                  experts, top, kind, normalize, groups, keep);
     RI_LAUNCH_CHECK("experts_route");
     return 0;
 }
 
-extern "C" int ri_experts_activate(void* out, const void* gu, int dtype, const float* dense, int tokens, int experts,
-                                   int ff, float limit, void* stream) {
+extern "C" int ri_experts_route(int32_t* ids, float* weights, float* dense, const float* z, const float* correction,
+                                int tokens, int experts, int top, void* stream) {
+    return ri_experts_route_general(ids, weights, dense, nullptr, z, experts, correction, tokens, experts, experts, top,
+                                    ROUTE_SIGMOID, 1, 1, 1, stream);
+}
+
+extern "C" int ri_experts_activate_strided(void* out, const void* gu, int dtype, const float* dense, int dense_stride,
+                                           int tokens, int experts, int ff, float limit, void* stream) {
+    RI_REQUIRE(!dense || dense_stride >= experts, "experts_activate: weight rows of %d for %d experts", dense_stride, experts);
     RI_REQUIRE(tokens > 0 && experts >= 1 && experts <= 65535 && ff >= 1, "experts_activate: %d tokens, %d experts of %d",
                tokens, experts, ff);
     RI_REQUIRE(dtype == RI_F32 || dtype == RI_BF16, "experts_activate: dtype %d", dtype);
     const dim3 grid(tokens, experts);
     hipStream_t s = (hipStream_t)stream;
     if (dtype == RI_F32)
-        experts_activate_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)gu, dense, experts, ff, limit);
+        experts_activate_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)gu, dense, dense_stride, experts, ff, limit);
     else
-        experts_activate_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)gu, dense, experts, ff, limit);
+        experts_activate_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)gu, dense, dense_stride, experts, ff, limit);
     RI_LAUNCH_CHECK("experts_activate");
+    return 0;
+}
+
+extern "C" int ri_experts_activate(void* out, const void* gu, int dtype, const float* dense, int tokens, int experts,
+                                   int ff, float limit, void* stream) {
+    return ri_experts_activate_strided(out, gu, dtype, dense, experts, tokens, experts, ff, limit, stream);
+}
+
+// What a mixture of experts adds beside its routed experts' weighted sum, row by row, in float32:
+//   out[t] = routed[t] + own[t] * x[t] + gate[t] * shared[t]
+// own: the weight of the token's own row (the identity experts it chose), gate: the weight of an expert that every
+// token uses; both are columns of extra [tokens, 2].  routed may come as parts of a split product, added in order;
+// x and shared may be absent.
+template <typename TX, typename TS>
+__global__ void __launch_bounds__(256)
+experts_finish_kernel(float* __restrict__ out, const float* __restrict__ routed, int parts, size_t part_stride,
+                      const TX* __restrict__ x, const TS* __restrict__ shared, int shared_parts,
+                      const float* __restrict__ extra, int dim) {
+    const size_t at = (size_t)blockIdx.x * dim;
+    const float own = extra[(size_t)blockIdx.x * 2], gate = extra[(size_t)blockIdx.x * 2 + 1];
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        float v = routed[at + d];
+        for (int p = 1; p < parts; ++p) v += routed[p * part_stride + at + d];
+        if (x) v += own * to_f32(x[at + d]);
+        if (shared) {
+            float sv = to_f32(shared[at + d]);
+            for (int p = 1; p < shared_parts; ++p) sv += to_f32(shared[p * part_stride + at + d]);
+            v += gate * sv;
+        }
+        out[at + d] = v;
+    }
+}
+
+extern "C" int ri_experts_finish(float* out, const float* routed, int parts, const void* x, int x_dtype, const void* shared,
+                                 int shared_dtype, int shared_parts, const float* extra, int tokens, int dim, void* stream) {
+    RI_REQUIRE(tokens > 0 && dim > 0 && parts >= 1 && shared_parts >= 1 && extra && routed, "experts_finish: %d tokens of %d", tokens, dim);
+    RI_REQUIRE((x_dtype == RI_F32 || x_dtype == RI_BF16) && (shared_dtype == RI_F32 || shared_dtype == RI_BF16),
+               "experts_finish: dtypes %d and %d", x_dtype, shared_dtype);
+    RI_REQUIRE(shared_parts == 1 || shared_dtype == RI_F32, "experts_finish: parts of a product are float32");
+    hipStream_t s = (hipStream_t)stream;
+    const size_t stride = (size_t)tokens * dim;
+#define RI_GO(TX, TS) experts_finish_kernel<TX, TS><<<tokens, 256, 0, s>>>(out, routed, parts, stride, (const TX*)x, \
+                                                                          (const TS*)shared, shared_parts, extra, dim)
+    if (x_dtype == RI_F32) { if (shared_dtype == RI_F32) RI_GO(float, float); else RI_GO(float, bf16_t); }
+    else                   { if (shared_dtype == RI_F32) RI_GO(bf16_t, float); else RI_GO(bf16_t, bf16_t); }
+#undef RI_GO
+    RI_LAUNCH_CHECK("experts_finish");
     return 0;
 }

@@ -35,12 +35,16 @@ __global__ void gla_decay_kernel(float* __restrict__ z, const float* __restrict_
     z[e] = expf(log_sigmoid(z[e] + (z_bias ? z_bias[e % width] : 0.f)) * inv_tau);
 }
 
-template <typename TA, int RPT, int STAGE>
+// FIXED: the decay is one constant per head (head_decay[h]) instead of a number per token and key channel, and q, k
+// and v pass through silu on their way in (linear attention with a fixed decay); z is then not read.
+__device__ __forceinline__ float silu_of(float v) { return v / (1.0f + expf(-v)); }
+
+template <typename TA, int RPT, int STAGE, bool FIXED>
 __global__ void __launch_bounds__(256)
 gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, int q_off, int k_off, int v_off,
                 const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, float q_scale,
                 float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
-                int heads, int dim, int vdim, int nb, int z_is_decay) {
+                int heads, int dim, int vdim, int nb, int z_is_decay, const float* __restrict__ head_decay) {
     extern __shared__ float lds[];                           // two buffers of nb tokens: q, k, alpha (dim each), v (16)
     __shared__ float part[2][GLA_MAX_NB][4][GLA_COLS];       // the wavefronts' shares of o_t, two blocks in flight
     const int b = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * GLA_COLS;
@@ -83,7 +87,7 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
             const TA* x = proj + (size_t)tok * row + h * dim + i;
             rq[j] = to_f32(x[q_off]);
             rk[j] = to_f32(x[k_off]);
-            rz[j] = z[((size_t)tok * heads + h) * dim + i];
+            if (!FIXED) rz[j] = z[((size_t)tok * heads + h) * dim + i];
         }
 #pragma unroll
         for (int j = 0; j < GLA_VSTAGE; ++j) {
@@ -100,15 +104,21 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
             if (tid + j * 256 < per) {
                 const int i = s_ch[j];
                 float* at = buf + (size_t)s_tok[j] * stride;
-                at[i] = rq[j] * q_scale;
-                at[dim + i] = rk[j];
-                at[2 * dim + i] = z_is_decay ? rz[j] : expf(log_sigmoid(rz[j] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
+                if (FIXED) {
+                    at[i] = silu_of(rq[j]) * q_scale;
+                    at[dim + i] = silu_of(rk[j]);
+                    at[2 * dim + i] = head_decay[h];
+                } else {
+                    at[i] = rq[j] * q_scale;
+                    at[dim + i] = rk[j];
+                    at[2 * dim + i] = z_is_decay ? rz[j] : expf(log_sigmoid(rz[j] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
+                }
             }
         }
 #pragma unroll
         for (int j = 0; j < GLA_VSTAGE; ++j) {
             const int e = tid + j * 256;
-            if (e < nb * GLA_COLS) buf[(size_t)v_tok[j] * stride + 3 * dim + e % GLA_COLS] = rv[j];
+            if (e < nb * GLA_COLS) buf[(size_t)v_tok[j] * stride + 3 * dim + e % GLA_COLS] = FIXED ? silu_of(rv[j]) : rv[j];
         }
     };
     ask(t0);
@@ -190,10 +200,10 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
         if (live && j < rows_here) S[(size_t)(row0 + j) * vdim] = s[j];
 }
 
-extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
-                           float* z, const float* z_bias, float tau, float q_scale, float* state,
-                           const int32_t* cu_seqlens, const int32_t* slots, int seqs, int tokens, int heads, int dim,
-                           int vdim, void* stream) {
+static int gla_scan_go(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
+                       float* z, const float* z_bias, float tau, float q_scale, float* state,
+                       const int32_t* cu_seqlens, const int32_t* slots, int seqs, int tokens, int heads, int dim,
+                       int vdim, const float* head_decay, void* stream) {
     RI_REQUIRE(seqs > 0 && tokens >= seqs && heads > 0 && dim > 0 && vdim > 0, "gla_scan: %d sequences, %d heads of %d x %d", seqs, heads, dim, vdim);
     RI_REQUIRE(dim <= GLA_SLICES * GLA_MAX_ROWS, "gla_scan: key heads of %d exceed the kernel's %d", dim, GLA_SLICES * GLA_MAX_ROWS);
     RI_REQUIRE(heads <= 65535 && seqs <= 65535, "gla_scan: %d heads of %d sequences exceed one launch", heads, seqs);
@@ -215,7 +225,7 @@ extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row,
     const size_t lds = (size_t)2 * nb * (3 * dim + GLA_COLS) * sizeof(float);
     // a prompt: the decays of all its tokens in one pass, in place of z, before the walk
     int z_is_decay = 0;
-    if (tokens > seqs) {
+    if (tokens > seqs && !head_decay) {
         const long total = (long)tokens * heads * dim;
         RI_REQUIRE((total + 255) / 256 <= 2147483647L, "gla_scan: %ld decays exceed one launch", total);
         gla_decay_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(z, z_bias, 1.0f / tau, total, heads * dim);
@@ -224,22 +234,23 @@ extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row,
     // key heads of 64, 128, 256 or 512: a thread's rows are a fixed number, a multiple of 4, read 16 bytes at a time
     const int fixed = (dim == 64 || dim == 128 || dim == 256 || dim == 512) ? dim / GLA_SLICES : 0;
     // (more than 64 KB of dynamic LDS has to be asked for, once for every form of the kernel)
-#define RI_GLA_GO(T, V, G)                                                                                           \
+#define RI_GLA_GO(T, V, G, F)                                                                                        \
     if (lds > 48 * 1024) {                                                                                           \
         static bool asked = false;                                                                                   \
         if (!asked) {                                                                                                \
-            hipError_t e_ = hipFuncSetAttribute((const void*)gla_scan_kernel<T, V, G>,                               \
+            hipError_t e_ = hipFuncSetAttribute((const void*)gla_scan_kernel<T, V, G, F>,                             \
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);             \
             RI_REQUIRE(e_ == hipSuccess, "gla_scan: %s", hipGetErrorString(e_));                                     \
             asked = true;                                                                                            \
         }                                                                                                            \
     }                                                                                                                \
-    gla_scan_kernel<T, V, G><<<grid, 256, lds, s>>>(out, (const T*)proj, row, q_off, k_off, v_off, z, z_bias, 1.0f / tau,   \
-                                                 q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb, z_is_decay)
+    gla_scan_kernel<T, V, G, F><<<grid, 256, lds, s>>>(out, (const T*)proj, row, q_off, k_off, v_off, z, z_bias, 1.0f / tau,\
+                                                 q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb, z_is_decay, head_decay)
     // (blocks of up to 4 * 256 staged elements run with a quarter of the staging registers: more wavefronts a SIMD)
     const bool few = (long)nb * dim <= 4 * 256;
 #define RI_GLA_STAGE(T, R)                                                                                           \
-    if (few) { RI_GLA_GO(T, R, 4); } else { RI_GLA_GO(T, R, 16); }
+    if (head_decay) { if (few) { RI_GLA_GO(T, R, 4, true); } else { RI_GLA_GO(T, R, 16, true); } }                    \
+    else            { if (few) { RI_GLA_GO(T, R, 4, false); } else { RI_GLA_GO(T, R, 16, false); } }
 #define RI_GLA_ROWS(T)                                                                                               \
     switch (fixed) {                                                                                                 \
         case 4: RI_GLA_STAGE(T, 4) break;                                                                            \
@@ -254,6 +265,25 @@ extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row,
 #undef RI_GLA_GO
     RI_LAUNCH_CHECK("gla_scan");
     return 0;
+}
+
+extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
+                           float* z, const float* z_bias, float tau, float q_scale, float* state,
+                           const int32_t* cu_seqlens, const int32_t* slots, int seqs, int tokens, int heads, int dim,
+                           int vdim, void* stream) {
+    RI_REQUIRE(z, "gla_scan: no decay logits");
+    return gla_scan_go(out, proj, act_dtype, row, q_off, k_off, v_off, z, z_bias, tau, q_scale, state, cu_seqlens, slots,
+                       seqs, tokens, heads, dim, vdim, nullptr, stream);
+}
+
+// Linear attention with one fixed decay per head: S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with
+// q = silu(.) * q_scale, k = silu(.), v = silu(.) of the projection's columns; head_decay: float32 [heads].
+extern "C" int ri_decay_scan(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
+                             const float* head_decay, float q_scale, float* state, const int32_t* cu_seqlens,
+                             const int32_t* slots, int seqs, int tokens, int heads, int dim, int vdim, void* stream) {
+    RI_REQUIRE(head_decay, "decay_scan: no decays");
+    return gla_scan_go(out, proj, act_dtype, row, q_off, k_off, v_off, nullptr, nullptr, 1.0f, q_scale, state, cu_seqlens,
+                       slots, seqs, tokens, heads, dim, vdim, head_decay, stream);
 }
 
 // The scan's result per head through an RMS norm over vdim (one gain for all heads) and times silu(gate):

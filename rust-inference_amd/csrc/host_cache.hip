@@ -24,6 +24,7 @@ constexpr int32_t UNMAPPED = -1;
 
 struct PagePool {
     int num_pages, page_size, num_slots, max_pages_per_slot, window;   // window 0: every key stays
+    int keep_first = 0;                                                // the first tokens of a sequence stay behind a window too
     std::vector<int32_t> free_list;                                    // taken from the back: page 0 first
     std::vector<int32_t> owner;                                        // page -> slot, to catch double frees
     std::vector<int32_t> tables;                                       // [num_slots][max_pages_per_slot]
@@ -75,7 +76,8 @@ struct PagePool {
     int trim_behind_window(int slot, long length) {
         if (window <= 0) return 0;
         const long first_visible = std::max<long>(0, length - window + 1);   // of the next query, at `length`
-        for (long p = 0; p < first_visible / page_size && p < max_pages_per_slot; ++p)
+        const long kept_pages = ((long)keep_first + page_size - 1) / page_size;    // they hold the positions 0 .. keep_first - 1
+        for (long p = kept_pages; p < first_visible / page_size && p < max_pages_per_slot; ++p)
             if (give_back(slot, (int)p)) return 1;
         return 0;
     }
@@ -150,6 +152,11 @@ extern "C" int ri_pool_pages_needed(void* pool, int slot, long before, long n) {
     return ((PagePool*)pool)->pages_needed(slot, before, n);
 }
 extern "C" int ri_pool_reserve(void* pool, int slot, long before, long n) { return ((PagePool*)pool)->reserve(slot, before, n); }
+extern "C" int ri_pool_keep_first(void* pool, int tokens) {
+    RI_REQUIRE(pool && tokens >= 0, "a pool keeps %d first tokens", tokens);
+    ((PagePool*)pool)->keep_first = tokens;
+    return 0;
+}
 extern "C" int ri_pool_trim(void* pool, int slot, long length) { return ((PagePool*)pool)->trim_behind_window(slot, length); }
 extern "C" int ri_pool_release(void* pool, int slot) { return ((PagePool*)pool)->release(slot); }
 extern "C" int ri_pool_check(void* pool) { return ((PagePool*)pool)->check(); }

@@ -252,3 +252,113 @@ extern "C" int ri_qk_norm_temper_kv_write(void* qkv, int act_dtype, const float*
     RI_LAUNCH_CHECK("qk_norm_temper_kv_write");
     return 0;
 }
+
+// ------------------------------------------------------------------ rotation of neighbours, then the norm
+// Queries and keys of an attention whose rotation turns the neighbours (2i, 2i + 1) of the first rot_dims elements
+// of every head by pos * inv_freq[i] (the rest of the head passes), followed by a per-head RMS norm (with a gain of
+// `dim`, or without one: unit_norm), from a projection row that may hold more than this mixer's columns: q heads
+// at q_off, k heads at k_off, v heads at v_off of rows of row_len elements.  q in place, k and v into their pages.
+// Angle, sine and cosine, and the norm are float32; an element is rounded once.  One wavefront per (token, head),
+// a lane on pairs of neighbours; a prompt's values go a page at a time (values_to_pages_kernel).
+#define QP_PAIRS_PER_LANE 4     // head sizes up to 64 * 2 * 4
+
+template <typename TA, typename TC>
+__global__ void qk_pairs_norm_kv_write_kernel(
+    TA* __restrict__ proj, size_t row_len, int q_off, int k_off, int v_off, const float* __restrict__ inv_freq,
+    int rot_dims, const float* __restrict__ q_gain, const float* __restrict__ k_gain, int norm, float eps,
+    const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ page_table,
+    int table_width, TC* __restrict__ k_pages, TC* __restrict__ v_pages, int tokens, int heads, int kv_heads, int dim,
+    int vdim, int page_size, int write_values) {
+    const int lane = threadIdx.x & (RI_WAVE - 1);
+    const int all_heads = heads + 2 * kv_heads;
+    const long item = (long)blockIdx.x * (blockDim.x / RI_WAVE) + threadIdx.x / RI_WAVE;
+    if (item >= (long)tokens * all_heads) return;          // whole wavefront leaves together
+    const int t = (int)(item / all_heads), hh = (int)(item % all_heads);
+    TA* row = proj + (size_t)t * row_len;
+    const int pos = tok_pos[t];
+    const int page = page_table[(size_t)tok_seq[t] * table_width + pos / page_size];
+    if (hh >= heads + kv_heads) {
+        if (!write_values) return;
+        const int kvh = hh - heads - kv_heads;
+        const TA* x = row + v_off + (size_t)kvh * vdim;
+        TC* vt = v_pages + ((size_t)page * kv_heads + kvh) * page_size * vdim + pos % page_size;
+        for (int d = lane; d < vdim; d += RI_WAVE) from_f32(vt + (size_t)d * page_size, to_f32(x[d]));
+        return;
+    }
+    const bool is_q = hh < heads;
+    TA* x = row + (is_q ? q_off + (size_t)hh * dim : k_off + (size_t)(hh - heads) * dim);
+    float a[QP_PAIRS_PER_LANE], b[QP_PAIRS_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < QP_PAIRS_PER_LANE; ++j) {
+        const int i = 2 * (lane + j * RI_WAVE);              // this pair: elements i and i + 1
+        a[j] = i < dim ? to_f32(x[i]) : 0.f;
+        b[j] = i + 1 < dim ? to_f32(x[i + 1]) : 0.f;
+        if (i + 1 < rot_dims) {
+            float sn, cs;
+            sincosf((float)pos * inv_freq[i / 2], &sn, &cs);
+            const float u = a[j], v = b[j];
+            a[j] = u * cs - v * sn;
+            b[j] = v * cs + u * sn;
+        }
+        ss += a[j] * a[j] + b[j] * b[j];
+    }
+    const float* gain = is_q ? q_gain : k_gain;
+    const float f = norm ? 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps) : 1.0f;
+    TC* dst = is_q ? nullptr
+                   : k_pages + (((size_t)page * kv_heads + (hh - heads)) * page_size + pos % page_size) * dim;
+#pragma unroll
+    for (int j = 0; j < QP_PAIRS_PER_LANE; ++j) {
+        const int i = 2 * (lane + j * RI_WAVE);
+        if (i < dim) {
+            const float v = a[j] * f * (gain ? gain[i] : 1.0f);
+            if (is_q) from_f32(x + i, v); else from_f32(dst + i, v);
+        }
+        if (i + 1 < dim) {
+            const float v = b[j] * f * (gain ? gain[i + 1] : 1.0f);
+            if (is_q) from_f32(x + i + 1, v); else from_f32(dst + i + 1, v);
+        }
+    }
+}
+
+extern "C" int ri_qk_pairs_norm_kv_write(void* proj, int act_dtype, long row_len, int q_off, int k_off, int v_off,
+                                         const float* inv_freq, int rot_dims, const float* q_gain, const float* k_gain,
+                                         int norm, float eps, const int32_t* tok_pos, const int32_t* tok_seq,
+                                         const int32_t* cu_seqlens, int seqs, int max_new, const int32_t* page_table,
+                                         int table_width, void* k_pages, void* v_pages, int cache_dtype, int tokens,
+                                         int heads, int kv_heads, int dim, int vdim, int page_size, void* stream) {
+    RI_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0, "qk_pairs_norm_kv_write: tokens %d, heads %d, kv heads %d", tokens,
+               heads, kv_heads);
+    RI_REQUIRE(dim >= 1 && dim <= RI_WAVE * 2 * QP_PAIRS_PER_LANE && vdim >= 1, "qk_pairs_norm_kv_write: head sizes %d and %d",
+               dim, vdim);
+    RI_REQUIRE(rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && (rot_dims == 0 || inv_freq),
+               "qk_pairs_norm_kv_write: a rotation over %d of %d elements", rot_dims, dim);
+    RI_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + (long)heads * dim <= row_len &&
+               k_off + (long)kv_heads * dim <= row_len && v_off + (long)kv_heads * vdim <= row_len,
+               "qk_pairs_norm_kv_write: q, k, v at %d, %d, %d do not fit rows of %ld", q_off, k_off, v_off, row_len);
+    RI_REQUIRE(act_dtype == cache_dtype && (act_dtype == RI_F32 || act_dtype == RI_BF16),
+               "qk_pairs_norm_kv_write: activations (%d) and cache (%d) must share float32 or bfloat16", act_dtype, cache_dtype);
+    RI_REQUIRE(page_size > 0 && table_width > 0 && k_pages && v_pages, "qk_pairs_norm_kv_write: page geometry");
+    RI_REQUIRE((!q_gain && !k_gain) || norm, "qk_pairs_norm_kv_write: gains without a norm");
+    const long items = (long)tokens * (heads + 2 * kv_heads);
+    RI_REQUIRE((items + 3) / 4 <= 2147483647L, "qk_pairs_norm_kv_write: %ld heads exceed one launch", items);
+    RI_REQUIRE(!cu_seqlens || (seqs > 0 && max_new > 0), "qk_pairs_norm_kv_write: seqs %d, max_new %d", seqs, max_new);
+    hipStream_t s = (hipStream_t)stream;
+    // a prompt's values a page at a time, where the sizes allow it
+    const bool paged_values = cu_seqlens && max_new > 1 && page_size % QT_TOKENS == 0 && seqs <= 65535 && kv_heads <= 65535 &&
+                              (size_t)QT_TOKENS * (vdim + 1) * sizeof(float) <= 65536;
+#define RI_GO(T)                                                                                                        \
+    qk_pairs_norm_kv_write_kernel<T, T><<<(unsigned)((items + 3) / 4), 256, 0, s>>>(                                      \
+        (T*)proj, (size_t)row_len, q_off, k_off, v_off, inv_freq, rot_dims, q_gain, k_gain, norm, eps, tok_pos, tok_seq,  \
+        page_table, table_width, (T*)k_pages, (T*)v_pages, tokens, heads, kv_heads, dim, vdim, page_size, !paged_values); \
+    if (paged_values) {                                                                                                 \
+        dim3 grid((max_new + QT_TOKENS - 2) / QT_TOKENS + 1, seqs, kv_heads);                                            \
+        values_to_pages_kernel<T, T><<<grid, 256, QT_TOKENS * (vdim + 1) * sizeof(float), s>>>(                           \
+            (const T*)proj, (size_t)row_len, (size_t)v_off, cu_seqlens, tok_pos, page_table, table_width, (T*)v_pages,    \
+            kv_heads, vdim, page_size);                                                                                 \
+    }
+    if (act_dtype == RI_F32) { RI_GO(float) } else { RI_GO(bf16_t) }
+#undef RI_GO
+    RI_LAUNCH_CHECK("qk_pairs_norm_kv_write");
+    return 0;
+}

@@ -95,6 +95,26 @@ _SIGNATURES = {
     "ri_add_bias": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "ri_finish_norm": [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ri_attention_kept": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int, c_void_p,
+                          c_void_p],
+    "ri_qk_pairs_norm_kv_write": [c_void_p, c_int, ctypes.c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                  c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p,
+                                  c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_decay_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p,
+                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_embed_scaled": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p],
+    "ri_branch_norm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_int, c_void_p,
+                           c_int, c_int, c_void_p],
+    "ri_gate_rows": [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                     c_void_p],
+    "ri_row_norm_gate": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_float, c_int,
+                         c_int, c_int, c_void_p],
+    "ri_experts_route_general": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                 c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_experts_activate_strided": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "ri_experts_finish": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int,
+                          c_void_p],
 }
 
 _fn = {}
@@ -152,6 +172,60 @@ def _opt(t, name: str, dtype=None, shape=None):
 
 
 # ---------------------------------------------------------------- row-wise
+GATE_SIGMOID, GATE_SILU = 0, 1
+
+
+def embed_scaled(table: torch.Tensor, ids: torch.Tensor, scale: float, act_dtype=None):
+    """float32 ``E[ids] * scale`` and, with ``act_dtype``, the same rows in that format (else None)."""
+    tokens, dim = ids.shape[0], table.shape[1]
+    out = torch.empty((tokens, dim), dtype=torch.float32, device=table.device)
+    act = torch.empty((tokens, dim), dtype=act_dtype, device=table.device) if act_dtype is not None else None
+    _call("ri_embed_scaled", _dev(out, "out"), _opt(act, "act"), code(act_dtype or torch.float32), _dev(table, "table"),
+          code(table.dtype), _dev(ids, "ids", torch.int32, (tokens,)), float(scale), tokens, dim, _stream())
+    return out, act
+
+
+def branch_norm_add(residual: torch.Tensor, y: torch.Tensor, gain, bias, eps: float, norm_kind: int, layer_scale,
+                    act_dtype=None):
+    """``residual += layer_scale * norm(y)`` in place (float32), the norm a layer norm (``NORM_LAYER``, with ``bias``) or an
+    RMS norm (``NORM_RMS``) over ``y``'s rows with ``gain``; ``y`` is ``[T, dim]`` or float32 ``[parts, T, dim]`` (added in
+    order).  With ``act_dtype`` the new residual is also returned in that format."""
+    rows, dim = residual.shape
+    parts = y.shape[0] if y.dim() == 3 else 1
+    if tuple(y.shape[-2:]) != (rows, dim):
+        raise ShapeError(f"a branch output of {list(y.shape)} for a residual of {list(residual.shape)}")
+    act = torch.empty((rows, dim), dtype=act_dtype, device=residual.device) if act_dtype is not None else None
+    _call("ri_branch_norm_add", _dev(residual, "residual", torch.float32), _opt(act, "act"), code(act_dtype or torch.float32),
+          _dev(y, "y"), code(y.dtype), parts, _dev(gain, "gain", torch.float32, (dim,)),
+          _opt(bias, "bias", torch.float32, (dim,)), float(eps), int(norm_kind),
+          _opt(layer_scale, "layer_scale", torch.float32, (dim,)), rows, dim, _stream())
+    return act
+
+
+def gate_rows(out: torch.Tensor, out_off: int, x: torch.Tensor, proj: torch.Tensor, g_off: int, scale: float,
+              kind: int = GATE_SIGMOID) -> None:
+    """``out[:, out_off : out_off + w] = scale * x * gate(proj[:, g_off : g_off + w])`` for ``x [T, w]``; the gate is a
+    sigmoid or silu; ``out`` and ``proj`` share a format.  ``proj`` None: no gate, the scaled copy alone."""
+    rows, width = x.shape
+    if out.shape[0] != rows or (proj is not None and (out.dtype != proj.dtype or proj.shape[0] != rows)):
+        raise ShapeError(f"gate_rows: out {list(out.shape)} {out.dtype}, x {list(x.shape)}, gates "
+                         f"{None if proj is None else list(proj.shape)}")
+    _call("ri_gate_rows", _dev(out, "out"), out.shape[1], int(out_off), _dev(x, "x"), code(x.dtype), _opt(proj, "proj"),
+          proj.shape[1] if proj is not None else 0, int(g_off), code(out.dtype), float(scale), int(kind), rows, width, _stream())
+
+
+def row_norm_gate(out: torch.Tensor, out_off: int, x: torch.Tensor, gain, eps: float, proj, g_off: int, scale: float,
+                  kind: int = GATE_SIGMOID) -> None:
+    """``out[:, out_off : out_off + w] = scale * x / sqrt(mean(x^2) + eps) * gain * gate(proj[:, g_off : g_off + w])``, the
+    mean over the whole row of ``x [T, w]`` float32; ``gain`` and ``proj`` may be None."""
+    rows, width = x.shape
+    if out.shape[0] != rows or (proj is not None and (proj.dtype != out.dtype or proj.shape[0] != rows)):
+        raise ShapeError(f"row_norm_gate: out {list(out.shape)}, x {list(x.shape)}")
+    _call("ri_row_norm_gate", _dev(out, "out"), out.shape[1], int(out_off), _dev(x, "x", torch.float32),
+          _opt(gain, "gain", torch.float32, (width,)), float(eps), _opt(proj, "proj"),
+          proj.shape[1] if proj is not None else 0, int(g_off), code(out.dtype), float(scale), int(kind), rows, width, _stream())
+
+
 def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     """float32 rows ``table[ids]``; ids int32 ``[T]``, already checked to be inside the table."""
     tokens, dim = ids.shape[0], table.shape[1]
@@ -304,22 +378,51 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, 
 
 
 def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, kv_heads: int, head_dim: int,
-              window: int | None, scale: float, softcap: float | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
+              window: int | None, scale: float, softcap: float | None = None, slopes: torch.Tensor | None = None,
+              keep_first: int = 0, sinks: torch.Tensor | None = None, q_off: int = 0) -> torch.Tensor:
     """Attention of every new token over its sequence's pages; q is the first ``H dh`` columns of ``qkv``.
+    With a window, ``keep_first`` first tokens of the sequence stay visible behind it; ``sinks`` (float32 ``[heads]``)
+    adds ``exp(sinks[h])`` to the denominator of head ``h``'s softmax.  ``q_off``: the queries' first column in ``qkv``'s rows
+    where it is not 0.
     The size of a value head is read from ``v_pages [pages, kv_heads, v_dim, page]``; with ``softcap`` a score
     ``s`` becomes ``softcap * tanh(s / softcap)`` before the softmax; with ``slopes`` (float32 ``[heads]``) the score of
     head ``h`` at position ``p`` for the key at ``j`` then loses ``slopes[h] * (p - j)``."""
     tokens, stride = qkv.shape
+    if q_off < 0 or q_off + heads * head_dim > stride:
+        raise ShapeError(f"attention: queries at column {q_off} of rows of {stride} for {heads} heads of {head_dim}")
     v_dim = v_pages.shape[2]
     if tuple(k_pages.shape[:2]) != tuple(v_pages.shape[:2]) or k_pages.shape[2] != v_pages.shape[3] or k_pages.shape[3] != head_dim:
         raise ShapeError(f"attention: key pages {list(k_pages.shape)} and value pages {list(v_pages.shape)} for heads of {head_dim}")
     out = torch.empty((tokens, heads * v_dim), dtype=qkv.dtype, device=qkv.device)
-    _call("ri_attention", _dev(out, "out"), _dev(qkv, "qkv"), code(qkv.dtype), stride, _dev(k_pages, "k_pages"),
+    _call("ri_attention_kept", _dev(out, "out"), _dev(qkv, "qkv") + int(q_off) * qkv.element_size(), code(qkv.dtype), stride, _dev(k_pages, "k_pages"),
           _dev(v_pages, "v_pages"), code(k_pages.dtype), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(tok_seq, "tok_seq", torch.int32, (tokens,)), _dev(page_table, "page_table", torch.int32),
           page_table.shape[1], tokens, heads, kv_heads, head_dim, v_dim, k_pages.shape[2], int(window or 0),
-          float(scale), float(softcap or 0.0), _opt(slopes, "slopes", torch.float32, (heads,)), _stream())
+          float(scale), float(softcap or 0.0), _opt(slopes, "slopes", torch.float32, (heads,)), int(keep_first or 0),
+          _opt(sinks, "sinks", torch.float32, (heads,)), _stream())
     return out
+
+
+def qk_pairs_norm_kv_write(proj, q_off: int, k_off: int, v_off: int, inv_freq, q_gain, k_gain, norm: bool, eps: float,
+                           tok_pos, tok_seq, page_table, k_pages, v_pages, heads: int, kv_heads: int, dim: int, vdim: int,
+                           cu_seqlens=None, max_new: int = 0) -> None:
+    """In place on the projection rows ``proj [T, row]`` (q heads at column ``q_off``, k heads at ``k_off``, v heads at
+    ``v_off``): the neighbours ``(2i, 2i + 1)`` of the first ``2 len(inv_freq)`` elements of every q and k head turn by
+    ``pos * inv_freq[i]``, then, with ``norm``, every head is divided by its root mean square (and multiplied by the
+    gains, where given); q stays in ``proj``, k and v go to their pages."""
+    tokens, row = proj.shape
+    pages, _, page_size, _ = k_pages.shape
+    seqs = cu_seqlens.shape[0] - 1 if cu_seqlens is not None else 0
+    rot = 0 if inv_freq is None else 2 * inv_freq.shape[0]
+    _call("ri_qk_pairs_norm_kv_write", _dev(proj, "proj"), code(proj.dtype), row, int(q_off), int(k_off), int(v_off),
+          _opt(inv_freq, "inv_freq", torch.float32), rot, _opt(q_gain, "q_gain", torch.float32, (dim,)),
+          _opt(k_gain, "k_gain", torch.float32, (dim,)), int(bool(norm)), float(eps),
+          _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _opt(cu_seqlens, "cu_seqlens", torch.int32), seqs, int(max_new),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1],
+          _dev(k_pages, "k_pages", proj.dtype, (pages, kv_heads, page_size, dim)),
+          _dev(v_pages, "v_pages", proj.dtype, (pages, kv_heads, vdim, page_size)), code(k_pages.dtype),
+          tokens, heads, kv_heads, dim, vdim, page_size, _stream())
 
 
 def qk_norm_temper_kv_write(qkv, q_gain, k_gain, eps: float, temper, tok_pos, tok_seq, page_table, k_pages, v_pages,
@@ -408,6 +511,23 @@ def gla_scan(proj, q_off: int, k_off: int, v_off: int, z, z_bias, tau: float, q_
     _call("ri_gla_scan", _dev(out, "out"), _dev(proj, "proj"), code(proj.dtype), row, q_off, k_off, v_off,
           _dev(z, "z", torch.float32, (tokens, heads * dim)), _opt(z_bias, "z_bias", torch.float32, (heads * dim,)),
           float(tau), float(q_scale), _dev(state, "state", torch.float32),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
+          seqs, tokens, heads, dim, vdim, _stream())
+    return out
+
+
+def decay_scan(proj, q_off: int, k_off: int, v_off: int, head_decay, q_scale: float, state, cu_seqlens, slots,
+               heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """Linear attention with one fixed decay per head over the new tokens of every sequence, from the state its slot
+    holds: ``S <- decay_h S + k v^T``, ``o = S^T q`` with ``q = silu(.) * q_scale``, ``k = silu(.)``, ``v = silu(.)`` of the
+    projection's columns at ``q_off``, ``k_off``, ``v_off``; ``head_decay`` float32 ``[heads]``; ``state`` float32
+    ``[slots, heads, dim, vdim]``, updated in place.  Returns float32 ``[T, heads * vdim]``."""
+    tokens, row = proj.shape
+    seqs = slots.shape[0]
+    out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=proj.device)
+    _call("ri_decay_scan", _dev(out, "out"), _dev(proj, "proj"), code(proj.dtype), row, int(q_off), int(k_off), int(v_off),
+          _dev(head_decay, "head_decay", torch.float32, (heads,)), float(q_scale),
+          _dev(state, "state", torch.float32, (state.shape[0], heads, dim, vdim)),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
           seqs, tokens, heads, dim, vdim, _stream())
     return out
@@ -555,6 +675,40 @@ def experts_route(z: torch.Tensor, correction: torch.Tensor, top: int):
     return ids, weights, dense
 
 
+ROUTE_SIGMOID, ROUTE_SOFTMAX = 0, 1
+
+
+def experts_route_general(z: torch.Tensor, correction: torch.Tensor, outs: int, experts: int, top: int, kind: int,
+                          normalize: bool, groups: int = 1, keep: int = 1):
+    """The general router from float32 logits ``z [T, >= outs]``: scores ``s`` are the sigmoid or the softmax over the
+    ``outs`` outputs (``experts`` real ones, then identity experts); the choice is by ``s + correction`` among the outputs of
+    the ``keep`` best of ``groups`` equal runs of neighbours (a group's score: its largest choice score); weights are the
+    chosen ``s``, over their sum with ``normalize``.  Returns ``ids``, ``weights`` ``[T, top]``, ``dense [T, outs]`` and
+    ``extra [T, 2]`` (the identity experts' weight; the sigmoid of column ``outs`` of ``z`` where it has one)."""
+    tokens, stride = z.shape
+    ids = torch.empty((tokens, top), dtype=torch.int32, device=z.device)
+    weights = torch.empty((tokens, top), dtype=torch.float32, device=z.device)
+    dense = torch.empty((tokens, outs), dtype=torch.float32, device=z.device)
+    extra = torch.empty((tokens, 2), dtype=torch.float32, device=z.device)
+    _call("ri_experts_route_general", _dev(ids, "ids"), _dev(weights, "weights"), _dev(dense, "dense"), _dev(extra, "extra"),
+          _dev(z, "z", torch.float32), stride, _dev(correction, "correction", torch.float32, (outs,)), tokens, outs, experts,
+          int(top), int(kind), int(bool(normalize)), int(groups), int(keep), _stream())
+    return ids, weights, dense, extra
+
+
+def experts_finish(routed: torch.Tensor, x, shared, extra: torch.Tensor) -> torch.Tensor:
+    """float32 ``routed + extra[:, 0] * x + extra[:, 1] * shared`` row by row; ``routed`` (float32) and ``shared`` may
+    be ``[parts, T, dim]`` (added in order); ``x`` and ``shared`` may be None."""
+    tokens, dim = routed.shape[-2:]
+    parts = routed.shape[0] if routed.dim() == 3 else 1
+    shared_parts = shared.shape[0] if shared is not None and shared.dim() == 3 else 1
+    out = torch.empty((tokens, dim), dtype=torch.float32, device=routed.device)
+    _call("ri_experts_finish", _dev(out, "out"), _dev(routed, "routed", torch.float32), parts, _opt(x, "x"),
+          code(x.dtype) if x is not None else F32, _opt(shared, "shared"), code(shared.dtype) if shared is not None else F32,
+          shared_parts, _dev(extra, "extra", torch.float32, (tokens, 2)), tokens, dim, _stream())
+    return out
+
+
 def experts_sort(ids: torch.Tensor, experts: int):
     """The assignments ``ids [T, top]`` sorted by expert and, inside an expert, by token: ``dest [T * top]`` (the row
     of assignment ``t * top + k``) and ``offsets [experts + 1]`` (where every expert's rows begin), int32."""
@@ -590,7 +744,9 @@ def experts_combine(y: torch.Tensor, dest: torch.Tensor, weights: torch.Tensor) 
 def experts_activate(gu: torch.Tensor, dense, ff: int, limit: float) -> torch.Tensor:
     """``dense[t, e] * g sigmoid(1.702 g) (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``
     for ``gu [T, E * 2 * ff]`` (every expert's gate then up); ``[T, E * ff]``, zero for experts not chosen.  ``dense``
-    None: rows of one expert each (``gu [T, 2 * ff]``), every weight 1."""
+    None: rows of one expert each (``gu [T, 2 * ff]``), every weight 1.  ``limit <= 0``: the plain gated form
+    ``silu(gate) * up``.  ``dense`` may have more columns than there are experts (a router with outputs that are no
+    experts): the first ``E`` are read."""
     if dense is None:
         tokens = gu.shape[0]
         out = torch.empty((tokens, ff), dtype=gu.dtype, device=gu.device)
@@ -598,12 +754,13 @@ def experts_activate(gu: torch.Tensor, dense, ff: int, limit: float) -> torch.Te
             raise ShapeError(f"gate|up rows are {list(gu.shape)} for experts of {ff}")
         _call("ri_experts_activate", _dev(out, "out"), _dev(gu, "gu"), code(gu.dtype), None, tokens, 1, ff, float(limit), _stream())
         return out
-    tokens, experts = dense.shape
-    if tuple(gu.shape) != (tokens, experts * 2 * ff):
-        raise ShapeError(f"gate|up rows are {list(gu.shape)} for {experts} experts of {ff}")
+    tokens, outs = dense.shape
+    experts = gu.shape[1] // (2 * ff)
+    if tuple(gu.shape) != (tokens, experts * 2 * ff) or experts > outs:
+        raise ShapeError(f"gate|up rows are {list(gu.shape)} for experts of {ff}, weights {list(dense.shape)}")
     out = torch.empty((tokens, experts * ff), dtype=gu.dtype, device=gu.device)
-    _call("ri_experts_activate", _dev(out, "out"), _dev(gu, "gu"), code(gu.dtype), _dev(dense, "dense", torch.float32),
-          tokens, experts, ff, float(limit), _stream())
+    _call("ri_experts_activate_strided", _dev(out, "out"), _dev(gu, "gu"), code(gu.dtype), _dev(dense, "dense", torch.float32),
+          outs, tokens, experts, ff, float(limit), _stream())
     return out
 
 

@@ -1,4 +1,5 @@
-from . import attention, block, delta, experts, feed_forward, gla, norm, position, streams, qwen3, zidepel, pisulorn  # noqa: F401  (registers the parts)
+from . import (attention, block, decay_attention, delta, experts, feed_forward, gla, norm, parallel, position, streams,
+               qwen3, zidepel, pisulorn, zakelorn)  # noqa: F401  (registers the parts)
 from .base import Embedding, FeedForward, Head, Mixer, Norm, Part, PositionEncoding
 from .block import PreNormBlock, ResidualStream
 from .context import StepContext

@@ -49,6 +49,18 @@ class GroupedQueryAttention(Mixer):
     ``q, k, v, o, q_norm, k_norm`` where they are not ``<prefix>q_proj.weight`` and so on.  A mixer with any of
     ``v_dim``, ``softcap`` or ``q_temper`` takes no position encoding; its q/k norm, temperature and cache write
     are one kernel (``ops.qk_norm_temper_kv_write``).
+
+    A third family, with a position encoding that turns neighbouring elements (``position`` of a kind whose
+    ``pairs`` is true, for instance ``"rotate_pairs"``): q and k are rotated first and normed afterwards,
+    ``qk_norm="unit"`` norms them without gains (a head divided by its root mean square); ``keep_first`` keeps
+    a sequence's first tokens visible behind the ``window`` (position ``i`` sees ``j <= i`` with ``i - j < window`` or
+    ``j < keep_first``; kept tokens keep their own positions); ``sinks`` reads one number per query head
+    (``names["sink"]``) whose exponential joins the softmax's denominator, with no key and no value, unscaled;
+    ``gate="sigmoid"`` multiplies the heads side by side by ``sigmoid(W_g h)`` (``names["g"]``, read from the mixer's own
+    input) before the output product.  Any of these sends the mixer through ``ops.qk_pairs_norm_kv_write``; value
+    heads of their own size are welcome there.  Such a mixer can also run beside another one on one input and one
+    output product (``parts.parallel.ParallelMixers``): ``in_matrix``, ``core`` and ``out_matrix`` are its three
+    steps taken apart.
     """
 
     links_norms = True
@@ -57,7 +69,7 @@ class GroupedQueryAttention(Mixer):
                  eps: float = 1e-6, position: PartSpec | None = None, window: int | None = None,
                  qkv_bias: bool = False, o_bias: bool = False, v_dim: int | None = None, scale: float | None = None,
                  softcap: float | None = None, q_temper: tuple | None = None, names: dict | None = None,
-                 distance_slopes: tuple | None = None):
+                 distance_slopes: tuple | None = None, keep_first: int = 0, sinks: bool = False, gate: str | None = None):
         if heads < 1 or kv_heads < 1 or heads % kv_heads:
             raise ConfigError(f"{heads} attention heads not divisible by {kv_heads} kv heads")
         if not 1 <= head_dim <= ops.MAX_HEAD_DIM:
@@ -82,7 +94,22 @@ class GroupedQueryAttention(Mixer):
             raise ConfigError(f"{len(self.distance_slopes)} distance slopes for {heads} heads")
         self.tempered = self.v_dim != head_dim or self.q_temper is not None or self.distance_slopes is not None
         self.position = build_part("position", position or PartSpec("none"))
-        if (self.tempered or self.softcap is not None) and (position is not None and position.kind != "none"):
+        self.keep_first, self.sinks, self.gate = int(keep_first or 0), bool(sinks), gate
+        if gate not in (None, "sigmoid", "silu"):
+            raise ConfigError(f"an output gate {gate!r} is neither 'sigmoid' nor 'silu'")
+        if self.keep_first < 0 or (self.keep_first and window is None):
+            raise ConfigError(f"{keep_first} first tokens kept behind a window of {window}")
+        # rotation of neighbours, unit norm, kept first tokens, sinks or a gate: the third family
+        self.paired = (getattr(self.position, "pairs", False) or qk_norm == "unit" or self.keep_first > 0 or self.sinks
+                       or gate is not None)
+        if self.paired and (self.q_temper is not None or qkv_bias or o_bias):
+            raise ConfigError("an attention with a rotation of neighbours, kept first tokens, sinks or a gate takes no "
+                              "query temperature and no biases")
+        if self.paired and position is not None and position.kind != "none" and not getattr(self.position, "pairs", False):
+            raise ConfigError("an attention with kept first tokens, sinks or a gate rotates neighbours or not at all")
+        if self.paired and head_dim > 512:
+            raise ConfigError(f"head_dim {head_dim}: the kernel that rotates neighbours takes up to 512")
+        if not self.paired and (self.tempered or self.softcap is not None) and (position is not None and position.kind != "none"):
             raise ConfigError("an attention with a score cap, a query temperature or value heads of their own size "
                               "takes no position encoding")
         if (self.tempered or self.softcap is not None) and (qkv_bias or o_bias):
@@ -90,8 +117,14 @@ class GroupedQueryAttention(Mixer):
                               "takes no biases")
         p = prefix
         self.names = {"q": p + "q_proj.weight", "k": p + "k_proj.weight", "v": p + "v_proj.weight",
-                      "o": p + "o_proj.weight", "q_norm": p + "q_norm.weight", "k_norm": p + "k_norm.weight"}
+                      "o": p + "o_proj.weight", "q_norm": p + "q_norm.weight", "k_norm": p + "k_norm.weight",
+                      "sink": p + "sink", "g": p + "g_proj.weight"}
         self.names.update(names or {})
+        self.unit_norm = qk_norm == "unit"
+        self.q_width, self.k_width, self.v_width = heads * head_dim, kv_heads * head_dim, kv_heads * self.v_dim
+        self.out_width = heads * self.v_dim
+        # the columns of this mixer's input product: q, k, v and, with a gate, g
+        self.in_width = self.q_width + self.k_width + self.v_width + (self.out_width if gate else 0)
 
     def tensors(self):
         p, d, dh, n = self.prefix, self.hidden, self.head_dim, self.names
@@ -101,9 +134,13 @@ class GroupedQueryAttention(Mixer):
             n["v"]: TensorSpec((self.kv_heads * self.v_dim, d), MATRIX),
             n["o"]: TensorSpec((d, self.heads * self.v_dim), MATRIX),
         }
-        if self.qk_norm:
+        if self.qk_norm and not self.unit_norm:
             t[n["q_norm"]] = TensorSpec((dh,), GAIN)
             t[n["k_norm"]] = TensorSpec((dh,), GAIN)
+        if self.sinks:
+            t[n["sink"]] = TensorSpec((self.heads,), GAIN)
+        if self.gate:
+            t[n["g"]] = TensorSpec((self.heads * self.v_dim, d), MATRIX)
         if self.qkv_bias:
             t[p + "q_proj.bias"] = TensorSpec((self.heads * dh,), BIAS)
             t[p + "k_proj.bias"] = TensorSpec((self.kv_heads * dh,), BIAS)
@@ -113,14 +150,26 @@ class GroupedQueryAttention(Mixer):
         t.update(self.position.tensors())
         return t
 
-    def bind(self, weights, rt):
+    def in_matrix(self, weights):
+        """The rows of this mixer's input product, ``[q; k; v]`` and, with a gate, ``g``."""
+        n = self.names
+        return torch.cat([weights[n[x]] for x in (("q", "k", "v", "g") if self.gate else ("q", "k", "v"))], 0)
+
+    def out_matrix(self, weights):
+        return weights[self.names["o"]]
+
+    def bind(self, weights, rt, alone: bool = True):
+        """``alone`` False: another part owns the products before and after (mixers side by side); this one binds
+        what its ``core`` needs."""
         self.rt = rt
         p, n = self.prefix, self.names
-        qkv = torch.cat([weights[n["q"]], weights[n["k"]], weights[n["v"]]], 0)
-        self.w_qkv = rt.pack(rt.place_matrix(qkv))
-        self.w_o = rt.pack(rt.place_matrix(weights[n["o"]]), parts_ok=(p + "o_proj.bias") not in weights)
-        self.q_gain = rt.place_gain(weights[n["q_norm"]]) if self.qk_norm else None
-        self.k_gain = rt.place_gain(weights[n["k_norm"]]) if self.qk_norm else None
+        if alone:
+            self.w_qkv = rt.pack(rt.place_matrix(self.in_matrix(weights)), always=self.gate is not None)
+            self.w_o = rt.pack(rt.place_matrix(weights[n["o"]]), parts_ok=(p + "o_proj.bias") not in weights)
+        gains = self.qk_norm and not self.unit_norm
+        self.q_gain = rt.place_gain(weights[n["q_norm"]]) if gains else None
+        self.k_gain = rt.place_gain(weights[n["k_norm"]]) if gains else None
+        self.sink = rt.place_gain(weights[n["sink"]]) if self.sinks else None
         self.b_qkv = self.b_o = None
         if self.qkv_bias:
             self.b_qkv = rt.place_gain(torch.cat([weights[p + n + "_proj.bias"] for n in "qkv"], 0))
@@ -170,7 +219,8 @@ class GroupedQueryAttention(Mixer):
         return self.rt.takes_tiled(self.w_qkv, m)
 
     def cache_need(self):
-        return KVNeed(self.kv_heads, self.head_dim, self.window, None if self.v_dim == self.head_dim else self.v_dim)
+        return KVNeed(self.kv_heads, self.head_dim, self.window, None if self.v_dim == self.head_dim else self.v_dim,
+                      self.keep_first or None)
 
     def forward(self, x, ctx, store, page_table, link=None):
         rt = self.rt
@@ -178,6 +228,12 @@ class GroupedQueryAttention(Mixer):
             qkv = rt.linear_packed(x, self.w_qkv)
             if self.b_qkv is not None:
                 ops.add_bias(qkv, self.b_qkv)
+        if self.paired:
+            proj = ops.as_rows(qkv)
+            heads = torch.empty((proj.shape[0], self.out_width), dtype=proj.dtype, device=proj.device)
+            self.core(proj, 0, ctx, store, page_table, heads, 0, 1.0)
+            with profiler.section(profiler.OUT_PROJECTION):
+                return rt.linear_packed(heads, self.w_o, out_dtype=torch.float32, parts_ok=True)
         if self.tempered or self.softcap is not None:
             return self.forward_tempered(qkv, ctx, store, page_table, link)
         self.position.apply(qkv, ctx, self.heads, self.kv_heads, self.head_dim)
@@ -216,6 +272,29 @@ class GroupedQueryAttention(Mixer):
         with profiler.section(profiler.ATTENTION):
             o = self.attend(qkv, ctx, store, page_table)
         return self.project_out(o, link)
+
+    def core(self, proj, col0: int, ctx, store, page_table, out, out_col: int, out_scale: float) -> None:
+        """The mixer between its two products: ``proj [T, row]`` holds this mixer's q, k, v (and g) from column
+        ``col0`` on; the rotated and normed q stay there, k and v go to the pages, and the heads' results, times the
+        gate and ``out_scale``, are written into the columns ``out_col ..`` of ``out``."""
+        q_at, k_at = col0, col0 + self.q_width
+        v_at = k_at + self.k_width
+        with profiler.section(profiler.QK_NORM_ROPE_APPEND):
+            ops.qk_pairs_norm_kv_write(proj, q_at, k_at, v_at, self.position.rotation_table(), self.q_gain, self.k_gain,
+                                       bool(self.qk_norm), self.eps, ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages,
+                                       store.v_pages, self.heads, self.kv_heads, self.head_dim, self.v_dim,
+                                       ctx.cu_seqlens, ctx.max_new)
+        with profiler.section(profiler.ATTENTION):
+            o = self.attend_kept(proj, col0, ctx, store, page_table)
+            ops.gate_rows(out, out_col, o, proj if self.gate else None, v_at + self.v_width, out_scale,
+                          ops.GATE_SILU if self.gate == "silu" else ops.GATE_SIGMOID)
+
+    def attend_kept(self, proj, q_at, ctx, store, page_table):
+        """The attention of the third family: window with kept first tokens, sinks, value heads of any size."""
+        slopes = getattr(self, "slopes", None)
+        return ops.attention(proj, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
+                             self.kv_heads, self.head_dim, self.window, self.scale, self.softcap, slopes,
+                             keep_first=self.keep_first, sinks=self.sink, q_off=q_at)
 
     def forward_tempered(self, qkv, ctx, store, page_table, link):
         """No rotation: per-head norm, query temperature and the write of k and v in one kernel, then the attention

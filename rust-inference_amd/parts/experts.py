@@ -30,19 +30,47 @@ class RoutedExperts(FeedForward):
 
     Tensors: ``<prefix>router [experts, hidden]``, ``<prefix>correction [experts]``, ``<prefix>e<i>.gate`` / ``.up``
     ``[ff, hidden]``, ``<prefix>e<i>.down [hidden, ff]``.
+
+    Other routers and experts, by parameter.  ``scores="softmax"``: ``s`` is the softmax over all of the router's
+    outputs.  ``normalize=False``: the weights are the chosen ``s`` themselves.  ``groups=(count, keep)``: the outputs
+    form ``count`` equal groups of neighbours, a group's score is its largest ``s + correction``, and only outputs of the
+    ``keep`` best groups can be chosen.  ``identity=n``: the router has ``n`` more outputs after the experts', which
+    stand for experts that hand the token's own row on (times the weight) and have no tensors; they are scored,
+    grouped and chosen like the others.  ``limit=None``: an expert is ``W_down (silu(W_gate h) (W_up h))``.
+    ``shared=ff``: one more expert of that width and form, ``<prefix>shared.gate`` / ``.up`` / ``.down``, runs for
+    every token and is added times ``sigmoid(W_sg h)``, one number a token (``<prefix>shared.sg [1, hidden]``; its row
+    rides as the last row of the router's matrix).
     """
 
-    def __init__(self, hidden: int, inter: int, experts: int, top: int, limit: float, prefix: str):
-        if not 1 <= top <= experts <= ops.EXPERTS_MAX:
-            raise ConfigError(f"the {top} best of {experts} experts: the router takes up to {ops.EXPERTS_MAX} experts")
-        if not limit > 0:
+    def __init__(self, hidden: int, inter: int, experts: int, top: int, limit: float | None, prefix: str,
+                 scores: str = "sigmoid", normalize: bool = True, groups: tuple | None = None, identity: int = 0,
+                 shared: int | None = None):
+        self.outs = experts + int(identity)
+        if not 1 <= top <= self.outs <= ops.EXPERTS_MAX or experts < 1:
+            raise ConfigError(f"the {top} best of {experts} experts and {identity} identity experts: the router takes up to "
+                              f"{ops.EXPERTS_MAX} outputs")
+        if limit is not None and not limit > 0:
             raise ConfigError(f"the experts' limit {limit} must be positive")
-        self.hidden, self.inter, self.experts, self.top, self.limit, self.prefix = hidden, inter, experts, top, float(limit), prefix
+        if scores not in ("sigmoid", "softmax"):
+            raise ConfigError(f"router scores {scores!r} are neither 'sigmoid' nor 'softmax'")
+        self.hidden, self.inter, self.experts, self.top, self.prefix = hidden, inter, experts, top, prefix
+        self.limit = float(limit) if limit is not None else 0.0          # 0: the plain gated form
+        self.scores, self.normalize, self.identity, self.shared = scores, bool(normalize), int(identity), shared
+        self.groups, self.keep = (int(groups[0]), int(groups[1])) if groups else (1, 1)
+        if self.outs % self.groups or not 1 <= self.keep <= self.groups or top > self.keep * (self.outs // self.groups):
+            raise ConfigError(f"{self.outs} router outputs in {self.groups} groups of which {self.keep} stay, for the {top} best")
+        # the router of the first designs: one kernel call and no extras
+        self.simple = (scores == "sigmoid" and self.normalize and self.groups == 1 and not self.identity and shared is None)
 
     def tensors(self):
         p, t = self.prefix, {}
-        t[p + "router"] = TensorSpec((self.experts, self.hidden), MATRIX)
-        t[p + "correction"] = TensorSpec((self.experts,), BIAS)
+        t[p + "router"] = TensorSpec((self.outs, self.hidden), MATRIX)
+        t[p + "correction"] = TensorSpec((self.outs,), BIAS)
+        if self.shared is not None:
+            t[p + "shared.gate"] = TensorSpec((self.shared, self.hidden), MATRIX)
+            t[p + "shared.up"] = TensorSpec((self.shared, self.hidden), MATRIX)
+            t[p + "shared.down"] = TensorSpec((self.hidden, self.shared), MATRIX)
+            t[p + "shared.sg"] = TensorSpec((1, self.hidden), MATRIX)
         for e in range(self.experts):
             t[f"{p}e{e}.gate"] = TensorSpec((self.inter, self.hidden), MATRIX)
             t[f"{p}e{e}.up"] = TensorSpec((self.inter, self.hidden), MATRIX)
@@ -52,7 +80,13 @@ class RoutedExperts(FeedForward):
     def bind(self, weights, rt):
         self.rt = rt
         p = self.prefix
-        self.w_router = rt.pack(rt.place_matrix(weights[p + "router"]))
+        router = weights[p + "router"]
+        if self.shared is not None:                       # the shared expert's gate: one more row of logits
+            router = torch.cat([router, weights[p + "shared.sg"].to(router.dtype)], 0)
+            self.w_shared_in = rt.pack(rt.place_matrix(torch.cat([weights[p + "shared.gate"], weights[p + "shared.up"]], 0)),
+                                       swiglu=True)
+            self.w_shared_down = rt.pack(rt.place_matrix(weights[p + "shared.down"]), parts_ok=True)
+        self.w_router = rt.pack(rt.place_matrix(router))
         self.correction = rt.place_gain(weights[p + "correction"])
         rows = []
         for e in range(self.experts):
@@ -71,27 +105,42 @@ class RoutedExperts(FeedForward):
     def forward(self, x, ctx):
         rt = self.rt
         with profiler.section(profiler.MLP):
-            z = rt.linear_packed(x, self.w_router, out_dtype=torch.float32)
-            ids, weights, dense = ops.experts_route(z, self.correction, self.top)
+            z = ops.as_rows(rt.linear_packed(x, self.w_router, out_dtype=torch.float32))
+            extra = None
+            if self.simple:
+                ids, weights, dense = ops.experts_route(z, self.correction, self.top)
+            else:
+                ids, weights, dense, extra = ops.experts_route_general(
+                    z, self.correction, self.outs, self.experts, self.top,
+                    ops.ROUTE_SOFTMAX if self.scores == "softmax" else ops.ROUTE_SIGMOID, self.normalize, self.groups, self.keep)
             tokens = z.shape[0]
             routed = (rt.dtype == torch.bfloat16 and not rt.invariant and self.top < self.experts
                       and self.hidden % 8 == 0 and self.inter % 8 == 0)
+            own = self.identity > 0                   # whether the identity experts' share is still to be added
             if routed and tokens * self.top < self.experts:
-                return ops.experts_few_tokens(rt.normed_now(x), self.w_gate_up.w, self.w_down.w, ids, weights, self.inter,
-                                              self.limit)
-            if (routed and tokens >= self.SORTED_MIN_TOKENS and not ctx.is_decode
+                y, own = ops.experts_few_tokens(rt.normed_now(x), self.w_gate_up.w, self.w_down.w, ids, weights, self.inter,
+                                                self.limit), False
+            elif (routed and tokens >= self.SORTED_MIN_TOKENS and not ctx.is_decode
                     and not torch.cuda.is_current_stream_capturing()):
-                return self.forward_sorted(rt.normed_now(x), ids, weights)
-            gu = ops.as_rows(rt.linear_packed(x, self.w_gate_up))
-            a = ops.experts_activate(gu, dense, self.inter, self.limit)
-            # float32 into the residual (or in parts that the stream's next read adds)
-            return rt.linear_packed(a, self.w_down, out_dtype=torch.float32, parts_ok=True)
+                y, own = self.forward_sorted(rt.normed_now(x), ids, weights), False
+            else:
+                gu = ops.as_rows(rt.linear_packed(x, self.w_gate_up))
+                a = ops.experts_activate(gu, dense, self.inter, self.limit)
+                # float32 into the residual (or in parts that the stream's next read adds)
+                y = rt.linear_packed(a, self.w_down, out_dtype=torch.float32, parts_ok=True)
+            if not own and self.shared is None:
+                return y
+            shared = None
+            if self.shared is not None:
+                act = rt.linear_packed(x, self.w_shared_in)
+                shared = rt.linear_packed(act, self.w_shared_down, out_dtype=torch.float32, parts_ok=True)
+            return ops.experts_finish(y, rt.normed_now(x) if own else None, shared, extra)
 
     def forward_sorted(self, x, ids, weights):
         """A prompt: every expert's tokens as rows side by side, two library products an expert, the weighted sum in
         float32.  The host reads how many rows every expert has (one wait a layer), which a captured step could not."""
         ff = self.inter
-        dest, offsets = ops.experts_sort(ids, self.experts)
+        dest, offsets = ops.experts_sort(ids, self.outs)
         rows = ops.experts_gather(x, dest, self.top)
         y = torch.empty_like(rows)
         starts = offsets.tolist()
@@ -101,4 +150,6 @@ class RoutedExperts(FeedForward):
                 gu = torch.mm(rows[a:b], self.w_gate_up.w[e * 2 * ff:(e + 1) * 2 * ff].t())
                 act = ops.experts_activate(gu, None, ff, self.limit)
                 torch.mm(act, self.w_down.w[:, e * ff:(e + 1) * ff].t(), out=y[a:b])
+        if self.identity and starts[self.outs] > starts[self.experts]:
+            y[starts[self.experts]:] = rows[starts[self.experts]:]        # identity experts: the token's own row
         return ops.experts_combine(y, dest, weights)

@@ -22,10 +22,11 @@ from .spec import ModelSpec
 
 @register_part("embedding", "table")
 class TokenEmbedding(Embedding):
-    """``h[t, :] = E[id_t, :]`` without scaling (the reference: src/ops/embedding.rs:10-42)."""
+    """``h[t, :] = E[id_t, :]`` without scaling (the reference: src/ops/embedding.rs:10-42), or, with ``scale``,
+    ``E[id_t, :] * scale`` in float32 (a head tied to the table reads the table itself, unscaled)."""
 
-    def __init__(self, vocab: int, dim: int, name: str):
-        self.vocab, self.dim, self.name = vocab, dim, name
+    def __init__(self, vocab: int, dim: int, name: str, scale: float = 1.0):
+        self.vocab, self.dim, self.name, self.scale = vocab, dim, name, float(scale)
 
     def tensors(self):
         return {self.name: TensorSpec((self.vocab, self.dim), MATRIX)}
@@ -35,9 +36,13 @@ class TokenEmbedding(Embedding):
         self.table = rt.place_matrix(weights[self.name])
 
     def forward(self, ctx):
+        if self.scale != 1.0:
+            return ops.embed_scaled(self.table, ctx.tokens, self.scale)[0]
         return ops.embed_gather(self.table, ctx.tokens)
 
     def bind_plain(self, weights):
+        if self.scale != 1.0:
+            raise ConfigError("a scaled embedding has no plain form")
         self.table_plain = weights[self.name].to(torch.float32).numpy()
 
     def plain(self, ctx):

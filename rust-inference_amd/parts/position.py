@@ -52,3 +52,31 @@ class NoPosition(PositionEncoding):
 
     def plain(self, heads, positions):
         return heads
+
+
+@register_part("position", "rotate_pairs")
+class RotatePairs(PositionEncoding):
+    """Rotary encoding over the first ``dims`` elements of a head, in neighbouring pairs: the elements ``(2i, 2i + 1)``
+    at position ``p`` turn by the angle ``p * base^(-2i / dims)`` (``i < dims / 2``); what lies behind ``dims`` passes
+    unchanged.  The frequencies are rounded to float32 once; angle, sine and cosine are float32 in the kernel.
+    ``pairs`` tells the mixer that neighbours turn (not the halves of a head): it then rotates before it norms."""
+
+    pairs = True
+
+    def __init__(self, head_dim: int, dims: int, base: float):
+        if dims % 2 or not 0 <= dims <= head_dim:
+            raise ConfigError(f"a rotation over {dims} of {head_dim} elements: an even number up to the head size")
+        if dims and not base > 0:
+            raise ConfigError(f"the rotation's base {base} must be positive")
+        self.head_dim, self.dims, self.base = head_dim, dims, float(base)
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.inv_freq = None
+        if self.dims:
+            i = torch.arange(self.dims // 2, dtype=torch.float64)
+            self.inv_freq = torch.pow(torch.tensor(self.base, dtype=torch.float64), -2.0 * i / self.dims) \
+                .to(torch.float32).to(rt.device).contiguous()
+
+    def rotation_table(self):
+        return self.inv_freq
