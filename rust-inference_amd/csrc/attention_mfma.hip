@@ -115,6 +115,7 @@ struct Columns {
     floatx4 o[NT][DH / 16];
     float m[NT], l[NT];
     int qpos[NT], lo[NT];         // the column's query position (-1: no such column) and first visible key
+    int keep;                     // keys before this position stay visible although they lie before lo (0: none)
     // a cap c on the scores, s <- c tanh(s / c) with s = scale (q . k), applied to the raw products so that what
     // follows still multiplies by the scale: (q . k) <- cap_post * tanh((q . k) * cap_pre), cap_pre = scale / c,
     // cap_post = c / scale; both 0: no cap
@@ -168,7 +169,7 @@ __device__ __forceinline__ void scores_and_weights(Columns<DH, NT>& c, const Fra
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int key = key0 + e;
-                if (key > c.qpos[j] || key < c.lo[j]) s[e] = -INFINITY;
+                if (key > c.qpos[j] || (key < c.lo[j] && key >= c.keep)) s[e] = -INFINITY;
             }
         }
         float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
@@ -229,6 +230,7 @@ __device__ __forceinline__ void init_columns(Columns<DH, NT>& c) {
         c.l[j] = 0.f;
         c.qpos[j] = -1;
         c.lo[j] = 0;
+        c.keep = 0;
         c.cap_pre = c.cap_post = 0.f;
         c.bias[j] = 0.f;
         c.biased = false;
@@ -270,7 +272,7 @@ __device__ __forceinline__ void mask_scores(const Columns<DH, NT>& c, float (&s)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int key = key0 + e;
-            if (key > c.qpos[j] || key < c.lo[j]) s[j][e] = -INFINITY;
+            if (key > c.qpos[j] || (key < c.lo[j] && key >= c.keep)) s[j][e] = -INFINITY;
         }
 }
 
@@ -379,7 +381,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
                          const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ tok_pos,
                          const int32_t* __restrict__ page_table, int table_width, int heads, int kv_heads,
                          int window, float scale_log2, float cap_pre, float cap_post,
-                         const float* __restrict__ slopes, float inv_scale) {
+                         const float* __restrict__ slopes, float inv_scale, int keep_first,
+                         const float* __restrict__ sinks) {
     __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][PAGE * LdsPage<DH>::KS];
     __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][DH * LdsPage<DH>::VS];
     const int lane = threadIdx.x & 63;
@@ -401,12 +404,15 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
     c.cap_pre = cap_pre;
     c.cap_post = cap_post;
     c.biased = slopes != nullptr;
+    c.keep = window > 0 ? keep_first : 0;
     const int jg = lane >> 4;
+    float sink[NT];                                          // the column's sink in the exponents' units; -inf: none
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
         const int col = j * 16 + (lane & 15);
         const int tl = col / group, g = col - tl * group;
         if (slopes) c.bias[j] = slopes[kvh * group + g] * inv_scale;
+        sink[j] = sinks ? sinks[kvh * group + g] * 1.4426950408889634f : -INFINITY;
         if (tl < nt) {
             const int tok = t0 + tl;
             c.qpos[j] = tok_pos[tok];
@@ -426,6 +432,12 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
     const int min_qpos = (nt > 0 && full) ? tok_pos[t0] : -1;
     const int max_lo = (nt > 0 && window > 0) ? max(0, tok_pos[t0 + nt - 1] - window + 1) : 0;
     const int32_t* table = page_table + (long)b * table_width;
+    // The walk: the pages that hold kept first tokens and lie before the window's first page, then the window's
+    // pages.  Walk position W stands for the page RI_PG(W); a kept page is never taken for open (its keys from
+    // keep_first on are hidden), so it runs with the mask.
+    const int nk = c.keep > 0 ? min((c.keep + PAGE - 1) / PAGE, p_lo) : 0;
+    const int w_last = nk + p_hi - p_lo;
+#define RI_PG(W) ((W) < nk ? (W) : p_lo + (W) - nk)
 
     // What this thread carries of a page on its way from global memory to LDS: up to two 16-byte pieces
     // of the key page and of the value page, in plain registers.
@@ -448,9 +460,9 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
     // Every wavefront takes every page of the workgroup (those outside its own tokens' sight are masked
     // whole and add nothing), and the page numbers of the loads are clamped: no branch in a turn but the mask
     // and the move of the reference point, so that each half of a turn is one stretch of code to schedule.
-#define RI_TURN_LOADS(P)                                                                             \
-    RI_STAGE_LOAD(k_pages, sk0, sk1, table[min((P) + 2, p_hi)]);                                     \
-    RI_STAGE_LOAD(v_pages, sv0, sv1, table[min((P) + 1, p_hi)]);
+#define RI_TURN_LOADS(W)                                                                             \
+    RI_STAGE_LOAD(k_pages, sk0, sk1, table[RI_PG(min((W) + 2, w_last))]);                            \
+    RI_STAGE_LOAD(v_pages, sv0, sv1, table[RI_PG(min((W) + 1, w_last))]);
 #define RI_TURN_STORES(I)                                                                            \
     {                                                                                                \
         if (has0) stage_store_key<DH>(k_lds[((I) & 1) ^ 1], c0, sk0);                                \
@@ -459,8 +471,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
         if (TWO) stage_store_value<DH>(v_lds[(I) & 1], c0 + 256, sv1);                               \
         __syncthreads();                /* what arrived is in place; what was read may be overwritten */ \
     }
-#define RI_PAGE_OPEN(Q) ((Q) * PAGE + PAGE - 1 <= min_qpos && (Q) * PAGE >= max_lo)
-    RI_STAGE_LOAD(k_pages, sk0, sk1, table[p_lo]);
+#define RI_PAGE_OPEN(W) ((W) >= nk && RI_PG(W) * PAGE + PAGE - 1 <= min_qpos && RI_PG(W) * PAGE >= max_lo)
+    RI_STAGE_LOAD(k_pages, sk0, sk1, table[RI_PG(0)]);
     {
         if (has0) stage_store_key<DH>(k_lds[0], c0, sk0);
         if (TWO) stage_store_key<DH>(k_lds[0], c0 + 256, sk1);
@@ -468,29 +480,29 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
     __syncthreads();
     float s_cur[NT][8], ref[NT], m_new[NT];
     {                                                        // turn 0: the first page's scores and maxima
-        RI_TURN_LOADS(p_lo - 1);
+        RI_TURN_LOADS(-1);
         Frag kf[2][DH / 32];
         key_frags_from_lds<DH>(kf, k_lds[0], lane);
-        scores_of<DH, NT>(c, kf, s_cur, p_lo, lane);
-        if (!RI_PAGE_OPEN(p_lo)) mask_scores<DH, NT>(c, s_cur, p_lo, lane);
+        scores_of<DH, NT>(c, kf, s_cur, RI_PG(0), lane);
+        if (!RI_PAGE_OPEN(0)) mask_scores<DH, NT>(c, s_cur, RI_PG(0), lane);
         maxima_with<DH, NT>(c, s_cur, m_new, scale_log2);
         move_reference<DH, NT>(c, m_new, ref);
         RI_TURN_STORES(0);
     }
     // A turn with the next page open to every column of the wavefront has no mask in it; pages are open in
     // one stretch (behind the window's edge, before the diagonal), so the turns come as three loops.
-    auto turn = [&](int p, auto masked) {
-        const int i = p - p_lo + 1;
+    auto turn = [&](int p, auto masked) {                    // p: the walk position of the page whose weights are due
+        const int i = p + 1;
         RI_TURN_LOADS(p);
         Frag w[NT];
         float s_next[NT][8];
         {
             Frag kf[2][DH / 32];
             key_frags_from_lds<DH>(kf, k_lds[i & 1], lane);
-            scores_of<DH, NT>(c, kf, s_next, p + 1, lane);
+            scores_of<DH, NT>(c, kf, s_next, RI_PG(p + 1), lane);
             weights_of<DH, NT>(c, s_cur, ref, w, scale_log2);
         }
-        if (decltype(masked)::value) mask_scores<DH, NT>(c, s_next, p + 1, lane);
+        if (decltype(masked)::value) mask_scores<DH, NT>(c, s_next, RI_PG(p + 1), lane);
         {
             Frag vf[DH / 16];
             value_frags_from_lds<DH>(vf, v_lds[(i & 1) ^ 1], lane);
@@ -504,12 +516,12 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
             for (int e = 0; e < 8; ++e) s_cur[j][e] = s_next[j][e];
         RI_TURN_STORES(i);
     };
-    int p = p_lo;
-    for (; p < p_hi && !RI_PAGE_OPEN(p + 1); ++p) turn(p, std::true_type());
-    for (; p < p_hi && RI_PAGE_OPEN(p + 1); ++p) turn(p, std::false_type());
-    for (; p < p_hi; ++p) turn(p, std::true_type());
+    int p = 0;
+    for (; p < w_last && !RI_PAGE_OPEN(p + 1); ++p) turn(p, std::true_type());
+    for (; p < w_last && RI_PAGE_OPEN(p + 1); ++p) turn(p, std::false_type());
+    for (; p < w_last; ++p) turn(p, std::true_type());
     {                                                        // the last page's weights and value product
-        const int i = p_hi - p_lo + 1;
+        const int i = w_last + 1;
         Frag w[NT], vf[DH / 16];
         weights_of<DH, NT>(c, s_cur, ref, w, scale_log2);
         value_frags_from_lds<DH>(vf, v_lds[(i & 1) ^ 1], lane);
@@ -519,6 +531,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
 #undef RI_TURN_STORES
 #undef RI_PAGE_OPEN
 #undef RI_STAGE_LOAD
+#undef RI_PG
     finish_columns<DH, NT>(c);
 
 #pragma unroll
@@ -526,7 +539,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
         const int col = j * 16 + (lane & 15);
         const int tl = col / group, g = col - tl * group;
         if (tl >= nt) continue;
-        const float inv = 1.0f / c.l[j];
+        // the sink joins the denominator alone: exp(sink - maximum), in the exponents' units (exp2 of -inf is 0)
+        const float inv = 1.0f / (c.l[j] + __builtin_amdgcn_exp2f(sink[j] - c.m[j]));
         bf16_t* op = out + ((long)(t0 + tl) * heads + kvh * group + g) * DH + jg * 4;
 #pragma unroll
         for (int dt = 0; dt < DH / 16; ++dt) {
@@ -1241,11 +1255,13 @@ static int prefill_tiles(int head_dim, int group, int max_new, int seqs, int kv_
     return nt;
 }
 
-extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_stride, const void* k_pages,
-                                         const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
-                                         const int32_t* page_table, int table_width, int seqs, int max_new,
-                                         int heads, int kv_heads, int head_dim, int page_size, int window,
-                                         float scale, float softcap, const float* slopes, void* stream) {
+extern "C" int ri_attention_prefill_kept_bf16(void* out, const void* qkv, int q_stride, const void* k_pages,
+                                              const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
+                                              const int32_t* page_table, int table_width, int seqs, int max_new,
+                                              int heads, int kv_heads, int head_dim, int page_size, int window,
+                                              float scale, float softcap, const float* slopes, int keep_first,
+                                              const float* sinks, void* stream) {
+    RI_REQUIRE(keep_first >= 0, "attention_prefill_bf16: %d first tokens kept", keep_first);
     const float cap_pre = softcap > 0.f ? scale / softcap : 0.f, cap_post = softcap > 0.f ? softcap / scale : 0.f;
     RI_REQUIRE(scale > 0.f, "attention_prefill_bf16: the scale %g must be positive", (double)scale);
     if (check_common("attention_prefill_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
@@ -1265,7 +1281,7 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
         attn_prefill_mfma_kernel<DH, NT><<<grid, 256, 0, s>>>(                                                   \
             (bf16_t*)out, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,          \
             cu_seqlens, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, cap_pre,          \
-            cap_post, slopes, 1.f / scale);                                                                      \
+            cap_post, slopes, 1.f / scale, keep_first, sinks);                                                   \
         break;
     switch (head_dim * 8 + nt_tiles) {
         RI_PREFILL_CASE(32, 4)
@@ -1280,6 +1296,16 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
 #undef RI_PREFILL_CASE
     RI_LAUNCH_CHECK("attention_prefill_bf16");
     return 0;
+}
+
+extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_stride, const void* k_pages,
+                                         const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
+                                         const int32_t* page_table, int table_width, int seqs, int max_new,
+                                         int heads, int kv_heads, int head_dim, int page_size, int window,
+                                         float scale, float softcap, const float* slopes, void* stream) {
+    return ri_attention_prefill_kept_bf16(out, qkv, q_stride, k_pages, v_pages, cu_seqlens, tok_pos, page_table, table_width,
+                                          seqs, max_new, heads, kv_heads, head_dim, page_size, window, scale, softcap, slopes,
+                                          0, nullptr, stream);
 }
 
 extern "C" int ri_attention_decode_chunks(int max_len) { return (max_len + DECODE_CHUNK - 1) / DECODE_CHUNK; }

@@ -95,6 +95,9 @@ _SIGNATURES = {
     "ri_add_bias": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "ri_finish_norm": [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ri_attention_prefill_kept_bf16": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                       c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int,
+                                       c_void_p, c_void_p],
     "ri_attention_kept": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int, c_void_p,
                           c_void_p],
@@ -794,18 +797,23 @@ def mfma_attention_fits(dtype, head_dim: int, group: int, page_size: int, decode
 
 def attention_prefill_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_new: int,
                            heads: int, kv_heads: int, head_dim: int, window: int | None, scale: float,
-                           softcap: float | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
+                           softcap: float | None = None, slopes: torch.Tensor | None = None, keep_first: int = 0,
+                           sinks: torch.Tensor | None = None, q_off: int = 0) -> torch.Tensor:
     """Matrix-core attention for any number of new tokens per sequence (bfloat16, pages of 32).  With ``softcap`` a
     score ``s`` becomes ``softcap * tanh(s / softcap)`` before the softmax; with ``slopes`` (float32 ``[heads]``) head
-    ``h``'s score at position ``p`` for the key at ``j`` then loses ``slopes[h] * (p - j)``."""
+    ``h``'s score at position ``p`` for the key at ``j`` then loses ``slopes[h] * (p - j)``.  ``keep_first``, ``sinks`` and
+    ``q_off`` as in ``attention``."""
     tokens, stride = qkv.shape
+    if q_off < 0 or q_off + heads * head_dim > stride or q_off % 8:
+        raise ShapeError(f"attention: queries at column {q_off} of rows of {stride} for {heads} heads of {head_dim}")
     out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
-    _call("ri_attention_prefill_bf16", _dev(out, "out"), _dev(qkv, "qkv", torch.bfloat16), stride,
+    _call("ri_attention_prefill_kept_bf16", _dev(out, "out"), _dev(qkv, "qkv", torch.bfloat16) + 2 * int(q_off), stride,
           _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, max_new, heads, kv_heads, head_dim,
           k_pages.shape[2], int(window or 0), float(scale), float(softcap or 0.0),
-          _opt(slopes, "slopes", torch.float32, (heads,)), _stream())
+          _opt(slopes, "slopes", torch.float32, (heads,)), int(keep_first or 0), _opt(sinks, "sinks", torch.float32, (heads,)),
+          _stream())
     return out
 
 

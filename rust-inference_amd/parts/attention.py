@@ -292,6 +292,14 @@ class GroupedQueryAttention(Mixer):
     def attend_kept(self, proj, q_at, ctx, store, page_table):
         """The attention of the third family: window with kept first tokens, sinks, value heads of any size."""
         slopes = getattr(self, "slopes", None)
+        group = self.heads // self.kv_heads
+        if (self.v_dim == self.head_dim and proj.shape[1] % 8 == 0 and q_at % 8 == 0
+                and ops.mfma_attention_fits(proj.dtype, self.head_dim, group, store.page_size, False)):
+            # the matrix cores' prompt kernel, for single tokens too: a window's keys are few, and one wavefront
+            # walks them in the order of their pages whatever the step looks like
+            return ops.attention_prefill_bf16(proj, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos, page_table,
+                                              ctx.B, ctx.max_new, self.heads, self.kv_heads, self.head_dim, self.window,
+                                              self.scale, self.softcap, slopes, self.keep_first, self.sink, q_at)
         return ops.attention(proj, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
                              self.kv_heads, self.head_dim, self.window, self.scale, self.softcap, slopes,
                              keep_first=self.keep_first, sinks=self.sink, q_off=q_at)

@@ -75,14 +75,17 @@ def left_mixer(h, positions, w, p, m, eps, past=None):
     q = (h @ w[p + "q"].T).reshape(t, heads, d)
     k = (h @ w[p + "k"].T).reshape(t, kv, d)
     v = (h @ w[p + "v"].T).reshape(t, kv, dv)
-    q = rms_unit(rotate_pairs(q, positions, m["rot"]["dims"], m["rot"]["base"]), eps)
-    k = rms_unit(rotate_pairs(k, positions, m["rot"]["dims"], m["rot"]["base"]), eps)
+    rot = m.get("rot") or {"dims": 0, "base": 1.0}           # no rotation where the mixer names none
+    q = rms_unit(rotate_pairs(q, positions, rot["dims"], rot["base"]), eps)
+    k = rms_unit(rotate_pairs(k, positions, rot["dims"], rot["base"]), eps)
     if past is not None:
         k, v = np.concatenate([past[0], k]), np.concatenate([past[1], v])
         pos_k = np.concatenate([past[2], positions])
     else:
         pos_k = positions
-    o = sink_attention(q, k, v, positions, pos_k, m["scale"], m["mask"]["size"], m["mask"]["keep_first"], w[p + "sink"])
+    mask = m.get("mask") or {}                               # no mask: every earlier token is seen
+    size = mask.get("size") if mask.get("size") is not None else math.inf
+    o = sink_attention(q, k, v, positions, pos_k, m["scale"], size, mask.get("keep_first", 0), w[p + "sink"])
     o = o.reshape(t, heads * dv) * sigmoid(h @ w[p + "g"].T)
     return o @ w[p + "o"].T, (k, v, pos_k)
 

@@ -60,6 +60,7 @@ KERNEL_TESTS, SMALL_MACHINE = os.path.join(HERE, "test_kernels_gpu.py"), os.path
 SAMPLER_TESTS = os.path.join(HERE, "test_sampling_gpu.py")
 ZIDEPEL_TESTS = os.path.join(HERE, "test_zidepel_kernels_gpu.py")
 PISULORN_TESTS = os.path.join(HERE, "test_pisulorn_kernels_gpu.py")
+ZAKELORN_TESTS = os.path.join(HERE, "test_zakelorn_kernels_gpu.py")
 PISULORN_SELECT = "not two_equal_keys and not many_sequences"      # not the 1,300 keys and the 512 workgroups on the emulated matrix cores (minutes)
 SAMPLER_SELECT = "(same_token_as_the_plain_sampler or top_p_drops) and not large"     # not the 151,936 entries, not the engine
 
@@ -81,6 +82,7 @@ def runs():
         "sampler": _start([*PYTEST, *_workers(2), SAMPLER_TESTS, "-k", SAMPLER_SELECT]),
         "zidepel": _start([*PYTEST, *_workers(2), ZIDEPEL_TESTS]),
         "pisulorn": _start([*PYTEST, *_workers(2), PISULORN_TESTS, "-k", PISULORN_SELECT]),
+        "zakelorn": _start([*PYTEST, *_workers(2), ZAKELORN_TESTS]),
     }
     done = {}
     try:
@@ -122,6 +124,14 @@ def test_the_kernels_of_the_pisulorn_design_pass_on_the_cpu_build_between_guard_
     cores), the short convolutions with their tails, the gated delta rule's walk, the router, the experts of a few
     tokens and the sort of many, the tanh form of GELU."""
     _passed(runs["pisulorn"])
+
+
+def test_the_kernels_of_the_zakelorn_design_pass_on_the_cpu_build_between_guard_pages(runs):
+    """tests/test_zakelorn_kernels_gpu.py: the scaled embedding, the norm on a sublayer's output with its layer scale,
+    the rotation of neighbours with the unit norm and the cache write, the window with kept first tokens and sinks
+    (generic and on the emulated matrix cores), the gates, the linear attention with a fixed decay, the general
+    router and the experts' closing sum."""
+    _passed(runs["zakelorn"])
 
 
 @pytest.mark.parametrize("units, tests", [("sixteen units", 7), ("one unit", 61)])
