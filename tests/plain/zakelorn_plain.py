@@ -191,7 +191,7 @@ def forward(cfg, w, tokens, kept=None, start=0, layers_out=None, gaps_out=None):
     if kept is None:
         kept = [{} for _ in cfg["layers"]]
     positions = np.arange(start, start + len(tokens), dtype=np.float64)
-    x = w["embed"][np.asarray(tokens)] * cfg["embedding"]["scale"]
+    x = w["embed"][np.asarray(tokens)] * (cfg.get("embedding") or {}).get("scale", 1.0)
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}."
         y = parallel_mixer(x, positions, w, p + "mix.", layer["mixer"], eps, kept[i])
