@@ -2,7 +2,7 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--model 8b|0.6b|1.7b|4b|14b|32b]
-    python bench.py --design zidepel|pisulorn [--size 0.6b|8b] [--layers L]      # another workload: see design_comparison below
+    python bench.py --design zidepel|pisulorn|zakelorn [--size 0.6b|8b] [--layers L]      # another workload: see design_comparison below
 
 The default run has the layer sizes of Qwen3-8B with random weights
 (N(0, 0.02), norm gains 1 + N(0, 0.1), seed 2), a batch of 8 and prompts of 2,048 tokens in a
@@ -225,13 +225,53 @@ def pisulorn_like(q, layers, vocab, context):
             "layers": [(dense, moe, rec, moe)[i % 4] for i in range(layers)]}
 
 
+def zakelorn_like(q, layers, vocab, context):
+    """A Zakelorn configuration with the layer sizes of a Qwen3 one: the same width; in every layer softmax attention
+    with Qwen3's heads and head size, half of every head turned, a window of 1,024 keys that keeps the first 64, and
+    beside it linear attention with a quarter as many heads of the same size (over four layers the recurrent work of
+    the one delta-rule layer in four of the Pisulorn model); of every four layers the first has a dense feed-forward
+    half again as wide as Qwen3's, the second and the fourth eight experts of half Qwen3's width and two identity
+    experts in two groups of which one stays, two outputs a token, and a shared expert of a quarter of Qwen3's width;
+    the third has no feed-forward."""
+    d, h, g, dh, ff = q["hidden_size"], q["num_attention_heads"], q["num_key_value_heads"], q["head_dim"], q["intermediate_size"]
+    hr = max(1, h // 4)
+    mixer = {"left": {"heads": h, "kv_heads": g, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "rot": {"dims": dh // 2, "base": 1e6},
+                      "mask": {"size": 1024, "keep_first": 64}},
+             "right": {"heads": hr, "dim": dh, "vdim": dh, "decay": [1.0 - 2.0 ** -(3 + 5 * i / max(1, hr - 1)) for i in range(hr)]},
+             "left_scale": 0.7, "right_scale": 0.7}
+    dense = {"kind": "dense", "ff": ff * 3 // 2}
+    moe = {"kind": "moe", "expert": {"ff": ff // 2}, "shared": {"ff": ff // 4},
+           "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 2, "keep": 1}}}
+    return {"architecture": "Zakelorn", "vocab": vocab, "width": d, "norm": {"eps": 1e-5}, "embedding": {"scale": d ** 0.5},
+            "layers": [{"type": "parallel", "mixer": mixer, "mlp": (dense, moe, None, moe)[i % 4]} for i in range(layers)]}
+
+
 def design_comparison(args) -> int:
-    """`--design zidepel` or `--design pisulorn`: prefill and decode of a model of that design beside the Qwen3 model
+    """`--design zidepel`, `--design pisulorn` or `--design zakelorn`: prefill and decode of a model of that design beside the Qwen3 model
     of the same layer sizes (and, for Pisulorn, beside the Zidepel model of those sizes, the design closest to it)
     (random weights, `--layers` layers each, default 8, and a vocabulary of 32,768 for all so that the layers and not
     the output matrix are what is timed).  One JSON line; the default workload and its line are not touched."""
     sizes = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B}
     layers, vocab, context = args.layers or 8, 32768, args.context
+    if args.design == "zakelorn":
+        out = {"metric": "prefill and decode of the Zakelorn design beside Pisulorn and Qwen3 at equal layer sizes", "unit": "tok/s",
+               "n_gpus": 1, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids", "layers": layers,
+               "vocab": vocab, "steps": args.steps, "warmup": args.warmup, "sizes": {}}
+        for size in ([args.size] if args.size else ["0.6b", "8b"]):
+            q = dict(sizes[size], num_hidden_layers=layers, vocab_size=vocab, max_position_embeddings=context,
+                     tie_word_embeddings=False)
+            trio = {}
+            for name, cfg in (("qwen3", q), ("pisulorn", pisulorn_like(q, layers, vocab, context)),
+                              ("zakelorn", zakelorn_like(q, layers, vocab, context))):
+                b = ShapeBench(f"{name} at Qwen3-{size} layer sizes", cfg, vocab, 11, context, not args.no_graphs)
+                trio[name] = b.measure(args.prompt, (1, 8, 32), args.steps, args.warmup)
+                b.close()
+            out["sizes"][size] = trio
+        first = out["sizes"][next(iter(out["sizes"]))]
+        out["value"], out["higher_is_better"] = first["zakelorn"]["decode_b8"]["tok_s"], True
+        out["vs_pisulorn_decode_b8"] = round(first["zakelorn"]["decode_b8"]["tok_s"] / first["pisulorn"]["decode_b8"]["tok_s"], 3)
+        print(json.dumps(out))
+        return 0
     if args.design == "pisulorn":
         out = {"metric": "prefill and decode of the Pisulorn design beside Zidepel and Qwen3 at equal layer sizes", "unit": "tok/s",
                "n_gpus": 1, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids", "layers": layers,
@@ -285,7 +325,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the other models")
     ap.add_argument("--no-other-models", action="store_true", help="skip the Qwen3-0.6B and Qwen3-32B points")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel of a decode step from the host")
-    ap.add_argument("--design", choices=["zidepel", "pisulorn"], default=None,
+    ap.add_argument("--design", choices=["zidepel", "pisulorn", "zakelorn"], default=None,
                     help="another workload: this design beside Qwen3 at equal layer sizes (prefill, decode at batch 1, 8, 32)")
     ap.add_argument("--size", choices=["0.6b", "8b"], default=None, help="with --design: one of the two layer sizes only")
     args = ap.parse_args()

@@ -111,6 +111,11 @@ int ri_gla_step_fits(int dim, int vdim);
 int ri_gla_step(void* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off, int g_off,
                 const float* z, const float* z_bias, float tau, float q_scale, float* state, const int32_t* slots,
                 const float* gain, float eps, int seqs, int heads, int dim, int vdim, void* stream);
+// The step of the linear attention with a fixed decay per head (q, k, v through silu): float32 out [seqs, heads * vdim],
+// neither normed nor gated; head sizes as ri_gla_step_fits says.
+int ri_decay_step(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
+                  const float* head_decay, float q_scale, float* state, const int32_t* slots, int seqs, int heads, int dim,
+                  int vdim, void* stream);
 
 // The gated delta rule.  proj: [tokens, row] of act_dtype with the projections of q and k (kv_heads heads of dim each)
 // and v (heads heads of vdim) side by side from column q_off on: `channels` = 2 kv_heads dim + heads vdim columns.
@@ -204,6 +209,13 @@ int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q
                              const int32_t* page_table, int table_width, int seqs, int max_chunks, int heads,
                              int kv_heads, int head_dim, int page_size, int window, float scale, float softcap,
                              const float* slopes, int tiled_out, void* stream);
+// The same with the first keep_first keys visible behind a window and a number per head (sinks, may be NULL) whose
+// exponential joins the softmax's denominator; for steps that ri_attention_decode_streams says do not stream.
+int ri_attention_decode_kept_bf16(void* out, float* workspace, const void* qkv, int q_stride, const void* k_pages,
+                                  const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
+                                  const int32_t* page_table, int table_width, int seqs, int max_chunks, int heads,
+                                  int kv_heads, int head_dim, int page_size, int window, float scale, float softcap,
+                                  const float* slopes, int tiled_out, int keep_first, const float* sinks, void* stream);
 
 // tiled_out (both decode forms): the result [seqs, heads * head_dim] is written in the matrix cores' operand order
 // (see tiled_at in common.h) for the packed product that reads it.

@@ -561,7 +561,7 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
                         int heads, int kv_heads, int window, float scale_log2, int max_chunks, float cap_pre, float cap_post,
-                        const float* __restrict__ slopes, float inv_scale) {
+                        const float* __restrict__ slopes, float inv_scale, int keep_first) {
     __shared__ float o_lds[CW][DH * 17];           // [d * 17 + col]: no bank conflicts either way
     __shared__ float ml_lds[CW][2][16];
     const int lane = threadIdx.x & 63;
@@ -575,16 +575,19 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     const int qpos = tok_pos[tok];
     const int phys = max(page_table[(long)b * table_width + min(page, table_width - 1)], 0);   // not mapped: page 0, unused
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
-    if (chunk * (CW * PAGE) > qpos || chunk * (CW * PAGE) + CW * PAGE - 1 < lo) return;   // whole workgroup
+    const int keep = window > 0 ? keep_first : 0;             // keys before it stay visible behind the window
+    if (chunk * (CW * PAGE) > qpos || (chunk * (CW * PAGE) + CW * PAGE - 1 < lo && chunk * (CW * PAGE) >= keep))
+        return;                                              // whole workgroup
 
     // No load sits in a branch (the compiler counts loads in flight only along code without branches): a
     // wavefront without a page of its own fetches page `phys` all the same, a lane without a column the
     // group's last query, and neither is used.
-    const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
+    const bool has = page * PAGE <= qpos && (page * PAGE + PAGE - 1 >= lo || page * PAGE < keep);
     Columns<DH, 1> c;
     init_columns<DH, 1>(c);
     c.cap_pre = cap_pre;
     c.cap_post = cap_post;
+    c.keep = keep;
     const int jg = lane >> 4, col = lane & 15;
     if (slopes) {
         c.biased = true;
@@ -688,7 +691,8 @@ __device__ __forceinline__ void join_sum(const float* __restrict__ base, int cb,
 template <int DH, int PB>
 __global__ void __launch_bounds__(DH * PB)
 attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ tok_pos,
-                        int heads, int window, int max_chunks, int chunk_keys, int tiled) {
+                        int heads, int window, int max_chunks, int chunk_keys, int tiled, int keep_first,
+                        const float* __restrict__ sinks) {
     __shared__ float part_o[JOIN_PARTS][DH];
     __shared__ float part_ml[JOIN_PARTS][2];
     const int b = blockIdx.x, h = blockIdx.y;                       // token b is sequence b's one new token
@@ -701,22 +705,31 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
     const int parts = n <= JOIN_SERIAL ? 1 : JOIN_PARTS;
     const int per = (n + parts - 1) / parts;
     const float* base = ws + ((long)b * heads + h) * max_chunks * (DH + 2);
+    // the chunks of the kept first keys that lie before the window's first chunk: the first run takes them first
+    const int k_hi = window > 0 && keep_first > 0 ? min((keep_first - 1) / chunk_keys, c_lo - 1) : -1;
+    // a sink joins the denominator alone, exp(sink - maximum) in the exponents' units
+    const float sink = sinks ? sinks[h] * 1.4426950408889634f : -INFINITY;
     for (int p = tp; p < parts; p += PB) {
         const int c0 = c_lo + p * per, c1 = min(c_hi, c0 + per - 1);
+        const int k1 = p == 0 ? k_hi : -1;
         // Sixteen chunks' loads are asked for at once while the run has sixteen more, then four at a time, each
         // from an address pulled back into the run, and what lies past the run's end is left out where it would
         // be used: a loop that fetches a chunk and then uses it makes a trip to memory for every chunk.  The
         // sums are the same operations in the same order as such a loop's.
         float m = -INFINITY;
-        int cb = c0;
+        int cb = 0;
+        for (; cb <= k1; cb += 4) join_max<DH, 4>(base, cb, k1, m);
+        cb = c0;
         for (; cb + JOIN_SERIAL - 1 <= c1; cb += JOIN_SERIAL) join_max<DH, JOIN_SERIAL>(base, cb, c1, m);
         for (; cb <= c1; cb += 4) join_max<DH, 4>(base, cb, c1, m);
         float acc = 0.f, l = 0.f;
+        for (cb = 0; cb <= k1; cb += 4) join_sum<DH, 4>(base, cb, k1, d, m, acc, l);
         cb = c0;                                                    // always in chunk order
         for (; cb + JOIN_SERIAL - 1 <= c1; cb += JOIN_SERIAL) join_sum<DH, JOIN_SERIAL>(base, cb, c1, d, m, acc, l);
         for (; cb <= c1; cb += 4) join_sum<DH, 4>(base, cb, c1, d, m, acc, l);
         if (parts == 1) {                                           // the whole workgroup is here or nowhere
-            out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
+            out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] =
+                f32_to_bf16(acc / (l + exp2f(sink - m)));
             return;
         }
         part_o[p][d] = acc;
@@ -737,7 +750,8 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
         acc += part_o[p][d] * f;
         l += part_ml[p][1] * f;
     }
-    out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
+    out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] =
+        f32_to_bf16(acc / (l + exp2f(sink - m)));
 }
 
 // The join of up to CAP chunks (JOIN_SERIAL) with every load asked for at once, before the position is known:
@@ -748,7 +762,8 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
 template <int DH, int CAP>
 __global__ void __launch_bounds__(DH)
 attn_decode_join_small_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ tok_pos,
-                              int heads, int window, int max_chunks, int chunk_keys, int tiled) {
+                              int heads, int window, int max_chunks, int chunk_keys, int tiled, int keep_first,
+                              const float* __restrict__ sinks) {
     const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
     const float* base = ws + ((long)b * heads + h) * max_chunks * (DH + 2);
     float o[CAP], mc[CAP], lc[CAP];
@@ -768,31 +783,39 @@ attn_decode_join_small_kernel(bf16_t* __restrict__ out, const float* __restrict_
     // window < 0: the entries are not chunks at fixed places but the runs of the streaming kernel, all of
     // them written (an empty run as a maximum of -inf)
     const int c_lo = window < 0 ? 0 : lo / chunk_keys, c_hi = window < 0 ? max_chunks - 1 : qpos / chunk_keys;
+    // the chunks of the kept first keys count as well (those before the window's first chunk were written for them)
+    const int k_hi = window > 0 && keep_first > 0 ? min((keep_first - 1) / chunk_keys, c_hi) : -1;
+    const float sink = sinks ? sinks[h] * 1.4426950408889634f : -INFINITY;
     float m = -INFINITY;
 #pragma unroll
     for (int c = 0; c < CAP; ++c)
-        if (c >= c_lo && c <= c_hi) m = fmaxf(m, mc[c]);
+        if ((c >= c_lo && c <= c_hi) || c <= k_hi) m = fmaxf(m, mc[c]);
     float acc = 0.f, l = 0.f;
 #pragma unroll
     for (int c = 0; c < CAP; ++c) {                          // always in chunk order
-        if (c >= c_lo && c <= c_hi) {
+        if ((c >= c_lo && c <= c_hi) || c <= k_hi) {
             const float f = mc[c] == -INFINITY ? 0.f : exp2f(mc[c] - m);
             acc += o[c] * f;
             l += lc[c] * f;
         }
     }
-    out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
+    // a sink joins the denominator alone, exp(sink - maximum) in the exponents' units (exp2 of -inf is 0)
+    out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] =
+        f32_to_bf16(acc / (l + exp2f(sink - m)));
 }
 
 template <int DH>
 static void launch_join(bf16_t* out, const float* ws, const int32_t* tok_pos, int seqs, int heads, int window,
-                        int max_chunks, int tiled, hipStream_t s, int chunk_keys = DECODE_CHUNK) {
+                        int max_chunks, int tiled, hipStream_t s, int chunk_keys = DECODE_CHUNK, int keep_first = 0,
+                        const float* sinks = nullptr) {
     if (max_chunks <= JOIN_SERIAL)
         attn_decode_join_small_kernel<DH, JOIN_SERIAL><<<dim3(seqs, heads), DH, 0, s>>>(out, ws, tok_pos, heads, window,
-                                                                                     max_chunks, chunk_keys, tiled);
+                                                                                     max_chunks, chunk_keys, tiled,
+                                                                                     keep_first, sinks);
     else
         attn_decode_join_kernel<DH, JOIN_PARTS><<<dim3(seqs, heads), DH * JOIN_PARTS, 0, s>>>(out, ws, tok_pos, heads,
-                                                                                           window, max_chunks, chunk_keys, tiled);
+                                                                                           window, max_chunks, chunk_keys, tiled,
+                                                                                           keep_first, sinks);
 }
 
 // ------------------------------------------------------------------ decode: the new token's own q, k and v
@@ -1332,12 +1355,18 @@ extern "C" int ri_attention_decode_pieces(int seqs, int kv_heads, int heads, int
     return decode_pieces(seqs, kv_heads, heads / (kv_heads > 0 ? kv_heads : 1), max_chunks);
 }
 
-extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q_stride,
-                                        const void* k_pages, const void* v_pages, const int32_t* cu_seqlens,
-                                        const int32_t* tok_pos, const int32_t* page_table, int table_width, int seqs,
-                                        int max_chunks, int heads, int kv_heads, int head_dim, int page_size,
-                                        int window, float scale, float softcap, const float* slopes, int tiled_out,
-                                        void* stream) {
+// keep_first, sinks: the first keys that stay visible behind a window, and a number per head whose exponential joins
+// the softmax's denominator; only the kernels that work in chunks take them (where ri_attention_decode_streams says
+// the step streams, the caller takes the prompt kernel).
+extern "C" int ri_attention_decode_kept_bf16(void* out, float* workspace, const void* qkv, int q_stride,
+                                             const void* k_pages, const void* v_pages, const int32_t* cu_seqlens,
+                                             const int32_t* tok_pos, const int32_t* page_table, int table_width, int seqs,
+                                             int max_chunks, int heads, int kv_heads, int head_dim, int page_size,
+                                             int window, float scale, float softcap, const float* slopes, int tiled_out,
+                                             int keep_first, const float* sinks, void* stream) {
+    RI_REQUIRE(keep_first >= 0, "attention_decode_bf16: %d first tokens kept", keep_first);
+    RI_REQUIRE((keep_first == 0 && !sinks) || stream_splits(seqs, kv_heads, max_chunks) == 0,
+               "attention_decode_bf16: kept first tokens and sinks in a step that streams (%d sequences)", seqs);
     const float cap_pre = softcap > 0.f ? scale / softcap : 0.f, cap_post = softcap > 0.f ? softcap / scale : 0.f;
     RI_REQUIRE(scale > 0.f, "attention_decode_bf16: the scale %g must be positive", (double)scale);
     if (check_common("attention_decode_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
@@ -1383,8 +1412,9 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
         attn_decode_mfma_kernel<DH, CW><<<pgrid, CW * 64, 0, s>>>(                                                \
             workspace, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
             tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, all, cap_pre, cap_post,       \
-            slopes, 1.f / scale);                                                                                 \
-        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, all, tiled_out, s, CW * PAGE);     \
+            slopes, 1.f / scale, keep_first);                                                                     \
+        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, all, tiled_out, s, CW * PAGE,      \
+                        keep_first, sinks);                                                                       \
         break;
     switch (head_dim * 16 + DECODE_WAVES / pieces) {
         RI_DECODE_CASE(32, 8)
@@ -1400,6 +1430,17 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
 #undef RI_DECODE_CASE
     RI_LAUNCH_CHECK("attention_decode_bf16");
     return 0;
+}
+
+extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q_stride,
+                                        const void* k_pages, const void* v_pages, const int32_t* cu_seqlens,
+                                        const int32_t* tok_pos, const int32_t* page_table, int table_width, int seqs,
+                                        int max_chunks, int heads, int kv_heads, int head_dim, int page_size,
+                                        int window, float scale, float softcap, const float* slopes, int tiled_out,
+                                        void* stream) {
+    return ri_attention_decode_kept_bf16(out, workspace, qkv, q_stride, k_pages, v_pages, cu_seqlens, tok_pos, page_table,
+                                         table_width, seqs, max_chunks, heads, kv_heads, head_dim, page_size, window, scale,
+                                         softcap, slopes, tiled_out, 0, nullptr, stream);
 }
 
 // The decode attention of a layer from the raw fused projection (which is not changed): q/k norm, rotation,

@@ -404,6 +404,44 @@ experts_finish_kernel(float* __restrict__ out, const float* __restrict__ routed,
     }
 }
 
+// Rows whose width is a multiple of 4: a thread takes four neighbours of a row, a workgroup 1,024 columns, so that a
+// step of one token is many short workgroups and not one that walks the row.
+__device__ __forceinline__ float4 fin_ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 fin_ld4(const bf16_t* p) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xFFFF0000u), __uint_as_float(w.y << 16),
+                       __uint_as_float(w.y & 0xFFFF0000u));
+}
+
+template <typename TX, typename TS>
+__global__ void __launch_bounds__(256)
+experts_finish_vec_kernel(float* __restrict__ out, const float* __restrict__ routed, int parts, size_t part_stride,
+                          const TX* __restrict__ x, const TS* __restrict__ shared, int shared_parts,
+                          const float* __restrict__ extra, int dim) {
+    const int d = (blockIdx.y * 256 + threadIdx.x) * 4;
+    if (d >= dim) return;
+    const size_t at = (size_t)blockIdx.x * dim + d;
+    const float own = extra[(size_t)blockIdx.x * 2], gate = extra[(size_t)blockIdx.x * 2 + 1];
+    float4 v = fin_ld4(routed + at);
+    for (int p = 1; p < parts; ++p) {
+        const float4 w = fin_ld4(routed + p * part_stride + at);
+        v = make_float4(v.x + w.x, v.y + w.y, v.z + w.z, v.w + w.w);
+    }
+    if (x) {
+        const float4 w = fin_ld4(x + at);
+        v = make_float4(v.x + own * w.x, v.y + own * w.y, v.z + own * w.z, v.w + own * w.w);
+    }
+    if (shared) {
+        float4 sv = fin_ld4(shared + at);
+        for (int p = 1; p < shared_parts; ++p) {
+            const float4 w = fin_ld4(shared + p * part_stride + at);
+            sv = make_float4(sv.x + w.x, sv.y + w.y, sv.z + w.z, sv.w + w.w);
+        }
+        v = make_float4(v.x + gate * sv.x, v.y + gate * sv.y, v.z + gate * sv.z, v.w + gate * sv.w);
+    }
+    *reinterpret_cast<float4*>(out + at) = v;
+}
+
 extern "C" int ri_experts_finish(float* out, const float* routed, int parts, const void* x, int x_dtype, const void* shared,
                                  int shared_dtype, int shared_parts, const float* extra, int tokens, int dim, void* stream) {
     RI_REQUIRE(tokens > 0 && dim > 0 && parts >= 1 && shared_parts >= 1 && extra && routed, "experts_finish: %d tokens of %d", tokens, dim);
@@ -412,8 +450,14 @@ extern "C" int ri_experts_finish(float* out, const float* routed, int parts, con
     RI_REQUIRE(shared_parts == 1 || shared_dtype == RI_F32, "experts_finish: parts of a product are float32");
     hipStream_t s = (hipStream_t)stream;
     const size_t stride = (size_t)tokens * dim;
-#define RI_GO(TX, TS) experts_finish_kernel<TX, TS><<<tokens, 256, 0, s>>>(out, routed, parts, stride, (const TX*)x, \
-                                                                          (const TS*)shared, shared_parts, extra, dim)
+    const dim3 vgrid(tokens, (dim / 4 + 255) / 256);
+#define RI_GO(TX, TS)                                                                                                   \
+    if (dim % 4 == 0 && vgrid.y <= 65535)                                                                               \
+        experts_finish_vec_kernel<TX, TS><<<vgrid, 256, 0, s>>>(out, routed, parts, stride, (const TX*)x,                 \
+                                                                (const TS*)shared, shared_parts, extra, dim);            \
+    else                                                                                                                \
+        experts_finish_kernel<TX, TS><<<tokens, 256, 0, s>>>(out, routed, parts, stride, (const TX*)x,                    \
+                                                             (const TS*)shared, shared_parts, extra, dim)
     if (x_dtype == RI_F32) { if (shared_dtype == RI_F32) RI_GO(float, float); else RI_GO(float, bf16_t); }
     else                   { if (shared_dtype == RI_F32) RI_GO(bf16_t, float); else RI_GO(bf16_t, bf16_t); }
 #undef RI_GO

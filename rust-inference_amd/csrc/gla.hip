@@ -410,12 +410,15 @@ extern "C" int ri_gla_norm_gate(void* out, const float* o, const void* proj, int
 // in registers and stored; the slices' shares of o meet in LDS, where the head is normed and gated.
 #define GLA_STEP_ROWS 32
 
-template <typename TA, int ROWS>
+// FIXED (linear attention with one decay per head, head_decay[h]): q, k and v pass through silu, z is not read, and the
+// step's result leaves as it is, float32 in raw[seqs][heads * vdim]: its norm runs over all heads together, afterwards.
+template <typename TA, int ROWS, bool FIXED>
 __global__ void __launch_bounds__(256)
 gla_step_kernel(TA* __restrict__ out, const TA* __restrict__ proj, int row, int q_off, int k_off, int v_off, int g_off,
                 const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, float q_scale,
                 float* __restrict__ state, const int32_t* __restrict__ slots, const float* __restrict__ gain, float eps,
-                int heads, int dim, int vdim, int groups, int slices) {
+                int heads, int dim, int vdim, int groups, int slices, const float* __restrict__ head_decay,
+                float* __restrict__ raw) {
     __shared__ float qs[GLA_SLICES * GLA_MAX_ROWS], ks[GLA_SLICES * GLA_MAX_ROWS], as[GLA_SLICES * GLA_MAX_ROWS];
     __shared__ __attribute__((aligned(16))) float red[1024];                 // [slices][vdim]
     __shared__ float scratch[16];
@@ -430,12 +433,19 @@ gla_step_kernel(TA* __restrict__ out, const TA* __restrict__ proj, int row, int 
         s[j] = *reinterpret_cast<const float4*>(S + (size_t)min(row0 + j, dim - 1) * vdim);
     const TA* x = proj + (size_t)b * row;
     for (int i = tid; i < dim; i += 256) {
-        qs[i] = to_f32(x[q_off + h * dim + i]) * q_scale;
-        ks[i] = to_f32(x[k_off + h * dim + i]);
-        as[i] = expf(log_sigmoid(z[((size_t)b * heads + h) * dim + i] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
+        if (FIXED) {
+            qs[i] = silu_of(to_f32(x[q_off + h * dim + i])) * q_scale;
+            ks[i] = silu_of(to_f32(x[k_off + h * dim + i]));
+            as[i] = head_decay[h];
+        } else {
+            qs[i] = to_f32(x[q_off + h * dim + i]) * q_scale;
+            ks[i] = to_f32(x[k_off + h * dim + i]);
+            as[i] = expf(log_sigmoid(z[((size_t)b * heads + h) * dim + i] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
+        }
     }
     const TA* vx = x + v_off + h * vdim + 4 * g;
-    const float4 v = make_float4(to_f32(vx[0]), to_f32(vx[1]), to_f32(vx[2]), to_f32(vx[3]));
+    float4 v = make_float4(to_f32(vx[0]), to_f32(vx[1]), to_f32(vx[2]), to_f32(vx[3]));
+    if (FIXED) v = make_float4(silu_of(v.x), silu_of(v.y), silu_of(v.z), silu_of(v.w));
     __syncthreads();
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
@@ -460,8 +470,10 @@ gla_step_kernel(TA* __restrict__ out, const TA* __restrict__ proj, int row, int 
             for (int rr = 0; rr < slices; ++rr) t += red[rr * vdim + c];
             mine[e] = t;
             ss += t * t;
+            if (FIXED) raw[((size_t)b * heads + h) * vdim + c] = t;
         }
     }
+    if (FIXED) return;
     const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)vdim + eps);
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
@@ -497,9 +509,9 @@ extern "C" int ri_gla_step(void* out, const void* proj, int act_dtype, int row, 
     const dim3 grid(heads, seqs);
     const int rpt = (dim + slices - 1) / slices;
 #define RI_STEP_GO(T, ROWS)                                                                                          \
-    gla_step_kernel<T, ROWS><<<grid, 256, 0, s>>>((T*)out, (const T*)proj, row, q_off, k_off, v_off, g_off, z, z_bias,   \
+    gla_step_kernel<T, ROWS, false><<<grid, 256, 0, s>>>((T*)out, (const T*)proj, row, q_off, k_off, v_off, g_off, z, z_bias, \
                                                   1.0f / tau, q_scale, state, slots, gain, eps, heads, dim, vdim, groups, \
-                                                  slices)
+                                                  slices, nullptr, nullptr)
     if (act_dtype == RI_F32) {
         if (rpt <= 8) RI_STEP_GO(float, 8); else if (rpt <= 16) RI_STEP_GO(float, 16); else RI_STEP_GO(float, 32);
     } else {
@@ -507,5 +519,35 @@ extern "C" int ri_gla_step(void* out, const void* proj, int act_dtype, int row, 
     }
 #undef RI_STEP_GO
     RI_LAUNCH_CHECK("gla_step");
+    return 0;
+}
+
+// One new token a sequence of the linear attention with a fixed decay per head: the step on the state, the result as
+// it is, float32 out[seqs][heads * vdim] (row b of proj belongs to slots[b]).  Head sizes as ri_gla_step_fits says.
+extern "C" int ri_decay_step(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
+                             const float* head_decay, float q_scale, float* state, const int32_t* slots, int seqs,
+                             int heads, int dim, int vdim, void* stream) {
+    RI_REQUIRE(seqs > 0 && heads > 0 && ri_gla_step_fits(dim, vdim), "decay_step: %d sequences, %d heads of %d x %d", seqs,
+               heads, dim, vdim);
+    RI_REQUIRE(heads <= 65535 && seqs <= 65535, "decay_step: %d heads of %d sequences exceed one launch", heads, seqs);
+    RI_REQUIRE(head_decay && out && state && slots, "decay_step: decays, a state and an output are needed");
+    RI_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + heads * dim <= row && k_off + heads * dim <= row &&
+               v_off + heads * vdim <= row, "decay_step: q, k, v at %d, %d, %d do not fit rows of %d", q_off, k_off, v_off, row);
+    RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "decay_step: dtype %d", act_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    const int groups = vdim / 4, slices = 256 / groups;
+    const dim3 grid(heads, seqs);
+    const int rpt = (dim + slices - 1) / slices;
+#define RI_STEP_GO(T, ROWS)                                                                                          \
+    gla_step_kernel<T, ROWS, true><<<grid, 256, 0, s>>>(nullptr, (const T*)proj, row, q_off, k_off, v_off, 0, nullptr,   \
+                                                 nullptr, 1.0f, q_scale, state, slots, nullptr, 0.f, heads, dim, vdim,   \
+                                                 groups, slices, head_decay, out)
+    if (act_dtype == RI_F32) {
+        if (rpt <= 8) RI_STEP_GO(float, 8); else if (rpt <= 16) RI_STEP_GO(float, 16); else RI_STEP_GO(float, 32);
+    } else {
+        if (rpt <= 8) RI_STEP_GO(bf16_t, 8); else if (rpt <= 16) RI_STEP_GO(bf16_t, 16); else RI_STEP_GO(bf16_t, 32);
+    }
+#undef RI_STEP_GO
+    RI_LAUNCH_CHECK("decay_step");
     return 0;
 }

@@ -262,7 +262,9 @@ extern "C" int ri_qk_norm_temper_kv_write(void* qkv, int act_dtype, const float*
 // a lane on pairs of neighbours; a prompt's values go a page at a time (values_to_pages_kernel).
 #define QP_PAIRS_PER_LANE 4     // head sizes up to 64 * 2 * 4
 
-template <typename TA, typename TC>
+// HPW: heads a wavefront takes one after the other (all of one token, so that the angles' sines and cosines are made
+// once for them, and their loads are in flight together); a prompt runs with 4, single tokens with 1.
+template <typename TA, typename TC, int HPW>
 __global__ void qk_pairs_norm_kv_write_kernel(
     TA* __restrict__ proj, size_t row_len, int q_off, int k_off, int v_off, const float* __restrict__ inv_freq,
     int rot_dims, const float* __restrict__ q_gain, const float* __restrict__ k_gain, int norm, float eps,
@@ -270,53 +272,74 @@ __global__ void qk_pairs_norm_kv_write_kernel(
     int table_width, TC* __restrict__ k_pages, TC* __restrict__ v_pages, int tokens, int heads, int kv_heads, int dim,
     int vdim, int page_size, int write_values) {
     const int lane = threadIdx.x & (RI_WAVE - 1);
-    const int all_heads = heads + 2 * kv_heads;
+    const int all_heads = heads + (write_values ? 2 : 1) * kv_heads;   // without the values, only q and k heads are items
+    const int runs = (all_heads + HPW - 1) / HPW;                      // a token's heads in runs of HPW
     const long item = (long)blockIdx.x * (blockDim.x / RI_WAVE) + threadIdx.x / RI_WAVE;
-    if (item >= (long)tokens * all_heads) return;          // whole wavefront leaves together
-    const int t = (int)(item / all_heads), hh = (int)(item % all_heads);
+    if (item >= (long)tokens * runs) return;               // whole wavefront leaves together
+    const int t = (int)(item / runs), h0 = (int)(item % runs) * HPW;
     TA* row = proj + (size_t)t * row_len;
     const int pos = tok_pos[t];
     const int page = page_table[(size_t)tok_seq[t] * table_width + pos / page_size];
-    if (hh >= heads + kv_heads) {
-        if (!write_values) return;
-        const int kvh = hh - heads - kv_heads;
-        const TA* x = row + v_off + (size_t)kvh * vdim;
-        TC* vt = v_pages + ((size_t)page * kv_heads + kvh) * page_size * vdim + pos % page_size;
-        for (int d = lane; d < vdim; d += RI_WAVE) from_f32(vt + (size_t)d * page_size, to_f32(x[d]));
-        return;
-    }
-    const bool is_q = hh < heads;
-    TA* x = row + (is_q ? q_off + (size_t)hh * dim : k_off + (size_t)(hh - heads) * dim);
-    float a[QP_PAIRS_PER_LANE], b[QP_PAIRS_PER_LANE];
-    float ss = 0.f;
+    float a[HPW][QP_PAIRS_PER_LANE], b[HPW][QP_PAIRS_PER_LANE];
 #pragma unroll
-    for (int j = 0; j < QP_PAIRS_PER_LANE; ++j) {
-        const int i = 2 * (lane + j * RI_WAVE);              // this pair: elements i and i + 1
-        a[j] = i < dim ? to_f32(x[i]) : 0.f;
-        b[j] = i + 1 < dim ? to_f32(x[i + 1]) : 0.f;
-        if (i + 1 < rot_dims) {
-            float sn, cs;
-            sincosf((float)pos * inv_freq[i / 2], &sn, &cs);
-            const float u = a[j], v = b[j];
-            a[j] = u * cs - v * sn;
-            b[j] = v * cs + u * sn;
+    for (int u = 0; u < HPW; ++u) {
+        const int hh = h0 + u;
+        if (hh >= heads + kv_heads) continue;               // a value head, or none: below
+        const TA* x = row + (hh < heads ? q_off + (size_t)hh * dim : k_off + (size_t)(hh - heads) * dim);
+#pragma unroll
+        for (int j = 0; j < QP_PAIRS_PER_LANE; ++j) {
+            const int i = 2 * (lane + j * RI_WAVE);          // this pair: elements i and i + 1
+            a[u][j] = i < dim ? to_f32(x[i]) : 0.f;
+            b[u][j] = i + 1 < dim ? to_f32(x[i + 1]) : 0.f;
         }
-        ss += a[j] * a[j] + b[j] * b[j];
     }
-    const float* gain = is_q ? q_gain : k_gain;
-    const float f = norm ? 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps) : 1.0f;
-    TC* dst = is_q ? nullptr
-                   : k_pages + (((size_t)page * kv_heads + (hh - heads)) * page_size + pos % page_size) * dim;
+    float sn[QP_PAIRS_PER_LANE], cs[QP_PAIRS_PER_LANE];
 #pragma unroll
     for (int j = 0; j < QP_PAIRS_PER_LANE; ++j) {
         const int i = 2 * (lane + j * RI_WAVE);
-        if (i < dim) {
-            const float v = a[j] * f * (gain ? gain[i] : 1.0f);
-            if (is_q) from_f32(x + i, v); else from_f32(dst + i, v);
+        sn[j] = 0.f;
+        cs[j] = 1.f;
+        if (i + 1 < rot_dims) sincosf((float)pos * inv_freq[i / 2], &sn[j], &cs[j]);
+    }
+#pragma unroll
+    for (int u = 0; u < HPW; ++u) {
+        const int hh = h0 + u;
+        if (hh >= all_heads) continue;
+        if (hh >= heads + kv_heads) {                        // a value head: copied into its page, transposed
+            const int kvh = hh - heads - kv_heads;
+            const TA* x = row + v_off + (size_t)kvh * vdim;
+            TC* vt = v_pages + ((size_t)page * kv_heads + kvh) * page_size * vdim + pos % page_size;
+            for (int d = lane; d < vdim; d += RI_WAVE) from_f32(vt + (size_t)d * page_size, to_f32(x[d]));
+            continue;
         }
-        if (i + 1 < dim) {
-            const float v = b[j] * f * (gain ? gain[i + 1] : 1.0f);
-            if (is_q) from_f32(x + i + 1, v); else from_f32(dst + i + 1, v);
+        const bool is_q = hh < heads;
+        TA* x = row + (is_q ? q_off + (size_t)hh * dim : k_off + (size_t)(hh - heads) * dim);
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < QP_PAIRS_PER_LANE; ++j) {
+            const int i = 2 * (lane + j * RI_WAVE);
+            if (i + 1 < rot_dims) {
+                const float p = a[u][j], q = b[u][j];
+                a[u][j] = p * cs[j] - q * sn[j];
+                b[u][j] = q * cs[j] + p * sn[j];
+            }
+            ss += a[u][j] * a[u][j] + b[u][j] * b[u][j];
+        }
+        const float* gain = is_q ? q_gain : k_gain;
+        const float f = norm ? 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps) : 1.0f;
+        TC* dst = is_q ? nullptr
+                       : k_pages + (((size_t)page * kv_heads + (hh - heads)) * page_size + pos % page_size) * dim;
+#pragma unroll
+        for (int j = 0; j < QP_PAIRS_PER_LANE; ++j) {
+            const int i = 2 * (lane + j * RI_WAVE);
+            if (i < dim) {
+                const float v = a[u][j] * f * (gain ? gain[i] : 1.0f);
+                if (is_q) from_f32(x + i, v); else from_f32(dst + i, v);
+            }
+            if (i + 1 < dim) {
+                const float v = b[u][j] * f * (gain ? gain[i + 1] : 1.0f);
+                if (is_q) from_f32(x + i + 1, v); else from_f32(dst + i + 1, v);
+            }
         }
     }
 }
@@ -340,17 +363,24 @@ extern "C" int ri_qk_pairs_norm_kv_write(void* proj, int act_dtype, long row_len
                "qk_pairs_norm_kv_write: activations (%d) and cache (%d) must share float32 or bfloat16", act_dtype, cache_dtype);
     RI_REQUIRE(page_size > 0 && table_width > 0 && k_pages && v_pages, "qk_pairs_norm_kv_write: page geometry");
     RI_REQUIRE((!q_gain && !k_gain) || norm, "qk_pairs_norm_kv_write: gains without a norm");
-    const long items = (long)tokens * (heads + 2 * kv_heads);
-    RI_REQUIRE((items + 3) / 4 <= 2147483647L, "qk_pairs_norm_kv_write: %ld heads exceed one launch", items);
+    RI_REQUIRE(((long)tokens * (heads + 2 * kv_heads) + 3) / 4 <= 2147483647L, "qk_pairs_norm_kv_write: %ld heads exceed one launch",
+               (long)tokens * (heads + 2 * kv_heads));
     RI_REQUIRE(!cu_seqlens || (seqs > 0 && max_new > 0), "qk_pairs_norm_kv_write: seqs %d, max_new %d", seqs, max_new);
     hipStream_t s = (hipStream_t)stream;
     // a prompt's values a page at a time, where the sizes allow it
     const bool paged_values = cu_seqlens && max_new > 1 && page_size % QT_TOKENS == 0 && seqs <= 65535 && kv_heads <= 65535 &&
                               (size_t)QT_TOKENS * (vdim + 1) * sizeof(float) <= 65536;
-#define RI_GO(T)                                                                                                        \
-    qk_pairs_norm_kv_write_kernel<T, T><<<(unsigned)((items + 3) / 4), 256, 0, s>>>(                                      \
+    // (a wavefront takes four heads of a token where the launch still has 64 wavefronts a compute unit then: below
+    // that fewer, longer wavefronts do not pay)
+    const int all_heads = heads + (paged_values ? 1 : 2) * kv_heads;
+    const bool four = (long)tokens * all_heads >= 256L * ri_compute_units();
+    const long items = (long)tokens * ((all_heads + (four ? 3 : 0)) / (four ? 4 : 1));
+#define RI_PAIRS(T, HPW)                                                                                                \
+    qk_pairs_norm_kv_write_kernel<T, T, HPW><<<(unsigned)((items + 3) / 4), 256, 0, s>>>(                                 \
         (T*)proj, (size_t)row_len, q_off, k_off, v_off, inv_freq, rot_dims, q_gain, k_gain, norm, eps, tok_pos, tok_seq,  \
-        page_table, table_width, (T*)k_pages, (T*)v_pages, tokens, heads, kv_heads, dim, vdim, page_size, !paged_values); \
+        page_table, table_width, (T*)k_pages, (T*)v_pages, tokens, heads, kv_heads, dim, vdim, page_size, !paged_values)
+#define RI_GO(T)                                                                                                        \
+    if (four) RI_PAIRS(T, 4); else RI_PAIRS(T, 1);                                                                       \
     if (paged_values) {                                                                                                 \
         dim3 grid((max_new + QT_TOKENS - 2) / QT_TOKENS + 1, seqs, kv_heads);                                            \
         values_to_pages_kernel<T, T><<<grid, 256, QT_TOKENS * (vdim + 1) * sizeof(float), s>>>(                           \
@@ -359,6 +389,7 @@ extern "C" int ri_qk_pairs_norm_kv_write(void* proj, int act_dtype, long row_len
     }
     if (act_dtype == RI_F32) { RI_GO(float) } else { RI_GO(bf16_t) }
 #undef RI_GO
+#undef RI_PAIRS
     RI_LAUNCH_CHECK("qk_pairs_norm_kv_write");
     return 0;
 }

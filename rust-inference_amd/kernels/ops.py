@@ -64,6 +64,9 @@ _SIGNATURES = {
     "ri_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int,
                                  c_void_p],
+    "ri_attention_decode_kept_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int,
+                                      c_int, c_void_p, c_void_p],
     "ri_attention_decode_fused_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float,
                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                        c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
@@ -104,6 +107,8 @@ _SIGNATURES = {
     "ri_qk_pairs_norm_kv_write": [c_void_p, c_int, ctypes.c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                   c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p,
                                   c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_decay_step": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int,
+                      c_int, c_int, c_void_p],
     "ri_decay_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p,
                       c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_embed_scaled": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p],
@@ -536,6 +541,19 @@ def decay_scan(proj, q_off: int, k_off: int, v_off: int, head_decay, q_scale: fl
     return out
 
 
+def decay_step(proj, q_off: int, k_off: int, v_off: int, head_decay, q_scale: float, state, slots, heads: int, dim: int,
+               vdim: int) -> torch.Tensor:
+    """``decay_scan`` for one new token a sequence (row ``b`` of ``proj`` belongs to ``slots[b]``), where ``gla_step_fits``
+    says the head sizes are taken: the state's trip from memory and back in 16-byte pieces.  float32 ``[seqs, heads * vdim]``."""
+    seqs, row = proj.shape
+    out = torch.empty((seqs, heads * vdim), dtype=torch.float32, device=proj.device)
+    _call("ri_decay_step", _dev(out, "out"), _dev(proj, "proj"), code(proj.dtype), row, int(q_off), int(k_off), int(v_off),
+          _dev(head_decay, "head_decay", torch.float32, (heads,)), float(q_scale),
+          _dev(state, "state", torch.float32, (state.shape[0], heads, dim, vdim)), _dev(slots, "slots", torch.int32, (seqs,)),
+          seqs, heads, dim, vdim, _stream())
+    return out
+
+
 def gla_step_fits(dim: int, vdim: int) -> bool:
     """Whether ``gla_step`` takes these head sizes (host code only: it needs no GPU)."""
     return bool(_get("ri_gla_step_fits")(int(dim), int(vdim)))
@@ -832,24 +850,30 @@ def decode_attention_streams(seqs: int, kv_heads: int, max_len: int) -> bool:
 
 def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_len: int,
                           heads: int, kv_heads: int, head_dim: int, window: int | None, scale: float,
-                          tiled_out: bool = False, softcap: float | None = None, slopes: torch.Tensor | None = None):
+                          tiled_out: bool = False, softcap: float | None = None, slopes: torch.Tensor | None = None,
+                          keep_first: int = 0, sinks: torch.Tensor | None = None, q_off: int = 0):
     """Matrix-core attention for one new token per sequence; ``max_len`` bounds every sequence's length
     after this step (it sizes the grid and the workspace, not the result).  ``tiled_out``: the result as
-    ``TiledRows`` (at most 64 sequences).  ``softcap`` and ``slopes`` as in ``attention_prefill_bf16``."""
+    ``TiledRows`` (at most 64 sequences).  ``softcap`` and ``slopes`` as in ``attention_prefill_bf16``; ``keep_first``,
+    ``sinks`` and ``q_off`` as in ``attention`` (in steps for which ``decode_attention_streams`` is false)."""
     tokens, stride = qkv.shape
     if tokens != seqs:
         raise ShapeError(f"decode attention takes one token per sequence, got {tokens} tokens for {seqs} sequences")
+    if q_off < 0 or q_off + heads * head_dim > stride or q_off % 8:
+        raise ShapeError(f"attention: queries at column {q_off} of rows of {stride} for {heads} heads of {head_dim}")
     chunks = _get("ri_attention_decode_chunks")(int(max_len))      # the kernels' own chunk size
     out = (TiledRows.empty(tokens, heads * head_dim, qkv.device) if tiled_out else
            torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device))
     pieces = _get("ri_attention_decode_pieces")(int(seqs), int(kv_heads), int(heads), chunks)
     ws = torch.empty((seqs, heads, chunks * pieces, head_dim + 2), dtype=torch.float32, device=qkv.device)
-    _call("ri_attention_decode_bf16", _dev(out.data if tiled_out else out, "out"), _dev(ws, "workspace"), _dev(qkv, "qkv", torch.bfloat16), stride,
+    _call("ri_attention_decode_kept_bf16", _dev(out.data if tiled_out else out, "out"), _dev(ws, "workspace"),
+          _dev(qkv, "qkv", torch.bfloat16) + 2 * int(q_off), stride,
           _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, chunks, heads, kv_heads, head_dim,
           k_pages.shape[2], int(window or 0), float(scale), float(softcap or 0.0),
-          _opt(slopes, "slopes", torch.float32, (heads,)), int(tiled_out), _stream())
+          _opt(slopes, "slopes", torch.float32, (heads,)), int(tiled_out), int(keep_first or 0),
+          _opt(sinks, "sinks", torch.float32, (heads,)), _stream())
     return out
 
 

@@ -293,10 +293,19 @@ class GroupedQueryAttention(Mixer):
         """The attention of the third family: window with kept first tokens, sinks, value heads of any size."""
         slopes = getattr(self, "slopes", None)
         group = self.heads // self.kv_heads
-        if (self.v_dim == self.head_dim and proj.shape[1] % 8 == 0 and q_at % 8 == 0
-                and ops.mfma_attention_fits(proj.dtype, self.head_dim, group, store.page_size, False)):
-            # the matrix cores' prompt kernel, for single tokens too: a window's keys are few, and one wavefront
-            # walks them in the order of their pages whatever the step looks like
+        fits = self.v_dim == self.head_dim and proj.shape[1] % 8 == 0 and q_at % 8 == 0
+        if (fits and ctx.is_decode and not self.rt.invariant
+                and ops.mfma_attention_fits(proj.dtype, self.head_dim, group, store.page_size, True)
+                and not ops.decode_attention_streams(ctx.B, self.kv_heads, ctx.max_len)):
+            # one new token a sequence in a step that does not fill the machine: the keys in chunks side by side, then
+            # the join, which adds the kept keys' chunks and the sink
+            return ops.attention_decode_bf16(proj, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos, page_table,
+                                             ctx.B, ctx.max_len, self.heads, self.kv_heads, self.head_dim, self.window,
+                                             self.scale, softcap=self.softcap, slopes=slopes, keep_first=self.keep_first,
+                                             sinks=self.sink, q_off=q_at)
+        if fits and ops.mfma_attention_fits(proj.dtype, self.head_dim, group, store.page_size, False):
+            # the matrix cores' prompt kernel, also for the single tokens of a step that fills the machine: a
+            # wavefront walks a sequence's pages in their order
             return ops.attention_prefill_bf16(proj, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos, page_table,
                                               ctx.B, ctx.max_new, self.heads, self.kv_heads, self.head_dim, self.window,
                                               self.scale, self.softcap, slopes, self.keep_first, self.sink, q_at)

@@ -68,6 +68,7 @@ class DecayLinearAttention(Mixer):
             self.w_o = rt.pack(rt.place_matrix(weights[self.names["o"]]), parts_ok=True)
         self.gain = rt.place_gain(weights[self.names["norm"]])
         self.head_decay = torch.tensor(self.decay, dtype=torch.float32, device=rt.device)
+        self.step_fits = ops.gla_step_fits(self.dim, self.vdim)
 
     def cache_need(self):
         return StateNeed((self.heads, self.dim, self.vdim), torch.float32)
@@ -77,8 +78,13 @@ class DecayLinearAttention(Mixer):
         times ``out_scale``, are written into the columns ``out_col ..`` of ``out``."""
         hk, hv = self.qk_width, self.out_width
         with profiler.section(profiler.ATTENTION):
-            o = ops.decay_scan(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.cu_seqlens, ctx.slots,
-                               self.heads, self.dim, self.vdim)
+            if ctx.is_decode and self.step_fits and not self.rt.invariant:
+                # one new token a sequence: the state in 16-byte pieces, a workgroup a sequence and head
+                o = ops.decay_step(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.slots, self.heads,
+                                   self.dim, self.vdim)
+            else:
+                o = ops.decay_scan(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.cu_seqlens,
+                                   ctx.slots, self.heads, self.dim, self.vdim)
             ops.row_norm_gate(out, out_col, o, self.gain, self.eps, proj if self.gate else None, col0 + 2 * hk + hv, out_scale,
                               ops.GATE_SILU if self.gate == "silu" else ops.GATE_SIGMOID)
 

@@ -72,6 +72,8 @@ def test_the_embedding_times_a_constant(ops, act):
     rng = np.random.default_rng(0)
     table = bf16_round(rng.normal(size=(37, 52)))
     ids = [5, 0, 36, 5]
+    odd, _ = ops.embed_scaled(t(table[:, :51].copy(), torch.bfloat16), t(ids, torch.int32), 6.25, act)
+    close(odd, table[ids, :51] * 6.25, 1e-7)
     out, rows = ops.embed_scaled(t(table, torch.bfloat16), t(ids, torch.int32), 6.25, act)
     close(out, table[ids] * 6.25, 1e-7)
     assert (rows is None) == (act is None)
@@ -79,7 +81,9 @@ def test_the_embedding_times_a_constant(ops, act):
         close(rows, table[ids] * 6.25, BF16_OUT)
 
 
-@pytest.mark.parametrize("dim, rows, parts, act", [(52, 5, 1, None), (200, 3, 3, torch.bfloat16), (1030, 2, 1, torch.bfloat16)])
+@pytest.mark.parametrize("dim, rows, parts, act", [(52, 5, 1, None), (200, 3, 3, torch.bfloat16), (1030, 2, 1, torch.bfloat16),
+                                                   (1300, 2, 2, torch.bfloat16), (4096, 2, 4, torch.bfloat16), (5000, 1, 1, None),
+                                                   (8196, 1, 2, torch.bfloat16)])
 def test_the_norm_on_a_sublayers_output_with_the_layer_scale(ops, dim, rows, parts, act):
     """residual += ls * layernorm(y): a mean far from zero and a small spread, which a variance taken as the mean of
     the squares minus the squared mean would lose in float32."""
@@ -271,6 +275,34 @@ def test_matrix_core_attention_with_kept_first_tokens_and_sinks(ops, form, dh, h
     got = ops.attention_prefill_bf16(t(wide, torch.bfloat16), kp, vp, t(new_cu, torch.int32), t(pos, torch.int32), table,
                                      len(lens), int(counts.max()), heads, kv_heads, dh, window, 0.21, None, None, keep, t(sinks), 16)
     close(got, want[rows], BF16_OUT, form)
+    if form == "single tokens":                                # the same through the chunks side by side and their join
+        got = ops.attention_decode_bf16(t(wide, torch.bfloat16), kp, vp, t(new_cu, torch.int32), t(pos, torch.int32), table,
+                                        len(lens), max(lens), heads, kv_heads, dh, window, 0.21, keep_first=keep,
+                                        sinks=t(sinks), q_off=16)
+        close(got, want[rows], BF16_OUT, "chunks and join")
+
+
+def test_kept_keys_and_a_sink_in_the_join_of_thousands_of_keys(ops):
+    """5,000 keys (more chunks than the short join takes at once), a window of 300 and 40 kept keys of which one answers
+    loudly: the join adds the first chunk to the window's two, and the sink to the denominator."""
+    rng = np.random.default_rng(12)
+    T, dh, window, keep, heads = 5000, 64, 300, 40, 4
+    q, k, v = rng.normal(size=(1, heads, dh)) * 0.3, rng.normal(size=(T, 2, dh)) * 0.3, rng.normal(size=(T, 2, dh))
+    q[0, :, 5] = 4.0
+    k[keep - 1, :, 5] = k[keep, :, 5] = 3.0                   # the last kept key, and the first that is not
+    q, k, v = bf16_round(q), bf16_round(k), bf16_round(v)
+    sinks = np.array([-20.0, 0.0, 3.0, 12.0])
+    want = plain_attention(q, k, v, [T - 1], 1.0, window, keep, sinks).reshape(1, -1)
+    assert np.abs(want[0, :dh] - v[keep - 1, 0]).max() < 0.05 * np.abs(v[keep - 1, 0]).max()
+    assert np.abs(want[0, 3 * dh:]).max() < 0.6 * np.abs(want[0, :dh]).max()          # the large sink takes most of the weight
+    kp, vp, table = paged_batch(k, v, [T], 3)
+    row = t(q.reshape(1, -1), torch.bfloat16)
+    got = ops.attention_decode_bf16(row, kp, vp, t([0, 1], torch.int32), t([T - 1], torch.int32), table, 1, T, heads, 2, dh,
+                                    window, 1.0, keep_first=keep, sinks=t(sinks))
+    close(got, want, BF16_OUT, "chunks and join")
+    got = ops.attention_prefill_bf16(row, kp, vp, t([0, 1], torch.int32), t([T - 1], torch.int32), table, 1, 1, heads, 2, dh,
+                                     window, 1.0, None, None, keep, t(sinks))
+    close(got, want, BF16_OUT, "prompt kernel")
 
 
 @pytest.mark.parametrize("dh", [32, 64])
@@ -288,6 +320,11 @@ def test_keys_at_the_edges_of_window_and_kept_tokens_matrix_cores(ops, dh, windo
                                          t(rows, torch.int32), table, 1, len(rows), heads, 1, dh, window, 1.0, None, None, keep,
                                          t(sinks))
         close(got, want[rows], 4e-3, what)
+        if len(rows) == 1:
+            got = ops.attention_decode_bf16(t(q[rows].reshape(1, -1), torch.bfloat16), kp, vp, t([0, 1], torch.int32),
+                                            t(rows, torch.int32), table, 1, T, heads, 1, dh, window, 1.0, keep_first=keep,
+                                            sinks=t(sinks))
+            close(got, want[rows], 4e-3, what + ", chunks and join")
 
 
 def test_one_far_kept_key_among_hundreds(ops):
@@ -328,9 +365,14 @@ def test_the_gate_on_the_heads_and_the_norm_over_all_heads(ops, dtype):
     close(out[:, 8:8 + w], 0.6 * xd * P.sigmoid(proj[:, 60:60 + w]), tol, "gate")
     assert (f64(out[:, :8]) == 7).all() and (f64(out[:, 8 + w:]) == 7).all()
     x32 = x.astype(np.float32).astype(np.float64)
-    ops.row_norm_gate(out, 48, t(x), t(gain), 1e-5, t(proj, dtype), 3, 0.9)
-    close(out[:, 48:48 + w], 0.9 * P.rms_unit(x32, 1e-5) * gain * P.sigmoid(proj[:, 3:3 + w]), tol, "norm and gate")
-    assert (f64(out[:, 8 + w:48]) == 7).all() and (f64(out[:, 48 + w:]) == 7).all()
+    for g_off in (3, 12):                                     # columns that 16-byte loads do not take, and columns they do
+        ops.row_norm_gate(out, 52, t(x), t(gain), 1e-5, t(proj, dtype), g_off, 0.9)
+        close(out[:, 52:52 + w], 0.9 * P.rms_unit(x32, 1e-5) * gain * P.sigmoid(proj[:, g_off:g_off + w]), tol, "norm and gate")
+        assert (f64(out[:, 8 + w:52]) == 7).all() and (f64(out[:, 52 + w:]) == 7).all()
+    ops.gate_rows(out, 1, t(x, dtype), t(proj, dtype), 61, 0.6)              # odd columns: one element a thread
+    close(out[:, 1:1 + w], 0.6 * xd * P.sigmoid(proj[:, 61:61 + w]), tol, "gate at odd columns")
+    ops.gate_rows(out, 4, t(x, dtype), None, 0, 2.0)
+    close(out[:, 4:4 + w], 2.0 * xd, tol, "no gate")
 
 
 # ---------------------------------------------------------------- linear attention with a fixed decay
@@ -370,6 +412,37 @@ def test_decay_scan(ops, dtype, H, dk, dv, lens):
     close(got, want, 1e-5, "outputs")
     close(dev_state, want_state, 1e-5, "state")
     assert np.array_equal(f64(dev_state[1]), state[1])        # a slot that no sequence of the step has
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H, dk, dv, seqs", [(4, 12, 20, 3), (2, 64, 48, 1), (1, 100, 128, 2), (2, 128, 128, 5), (3, 33, 8, 2),
+                                             (1, 256, 16, 1), (2, 128, 64, 2)])
+def test_decay_step(ops, dtype, H, dk, dv, seqs):
+    """One new token a sequence on states that are not zero, at slots in another order: the step kernel where it takes
+    the head sizes, against the plain walk and against the scan."""
+    if not ops.gla_step_fits(dk, dv):
+        pytest.skip("head sizes that the scan takes for single tokens too")
+    rng = np.random.default_rng(H * 13 + dk)
+    before = 4
+    row = before + 2 * H * dk + 2 * H * dv
+    proj = rng.normal(size=(seqs, row)).astype(np.float32).astype(np.float64)
+    if dtype == torch.bfloat16:
+        proj = bf16_round(proj)
+    decay = np.concatenate([[1.0], rng.uniform(0.3, 0.999, size=H)])[:H].astype(np.float32).astype(np.float64)
+    slots = [4, 0, 2, 5, 1][:seqs]
+    state = (rng.normal(size=(6, H, dk, dv)) * 0.5).astype(np.float32).astype(np.float64)
+    want_state = state.copy()
+    q_at, k_at, v_at = before, before + H * dk, before + 2 * H * dk
+    want = plain_decay(proj, q_at, k_at, v_at, H, dk, dv, decay, [1] * seqs, slots, want_state)
+    dev_state = t(state)
+    got = ops.decay_step(t(proj, dtype), q_at, k_at, v_at, t(decay), 1.0, dev_state, t(slots, torch.int32), H, dk, dv)
+    close(got, want, 1e-5, "outputs")
+    close(dev_state, want_state, 1e-5, "state")
+    assert np.array_equal(f64(dev_state[3]), state[3])
+    scan_state = t(state)
+    scan = ops.decay_scan(t(proj, dtype), q_at, k_at, v_at, t(decay), 1.0, scan_state, t(np.arange(seqs + 1), torch.int32),
+                          t(slots, torch.int32), H, dk, dv)
+    close(got, f64(scan), 2e-6, "step against scan")
 
 
 def test_decay_scan_token_by_token_is_the_walk_in_blocks(ops):
@@ -433,9 +506,10 @@ def test_a_dropped_groups_outputs_lose_to_negative_choice_scores(ops):
     close(dense, [[0.05, 0.10, 0.0, 0.0]], 1e-5)
 
 
-def test_the_experts_closing_sum(ops):
+@pytest.mark.parametrize("dim", [40, 41, 2052])
+def test_the_experts_closing_sum(ops, dim):
     rng = np.random.default_rng(1)
-    T, dim = 6, 40
+    T = 6
     routed, shared = rng.normal(size=(3, T, dim)), rng.normal(size=(2, T, dim))
     x = bf16_round(rng.normal(size=(T, dim)))
     extra = rng.uniform(size=(T, 2))
