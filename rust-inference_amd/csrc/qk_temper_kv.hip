@@ -344,6 +344,63 @@ __global__ void qk_pairs_norm_kv_write_kernel(
     }
 }
 
+// A prompt with head sizes that 16-byte pieces divide (8 times a power of two, up to 512): a workgroup a token, a lane
+// on eight neighbours (four pairs) of a head, so that a wavefront takes 512 / dim heads at once; the four angles'
+// sines and cosines are made once a lane and serve every head of the token.  q in place, k into its page; the values
+// go a page at a time (values_to_pages_kernel).
+template <typename TA, typename TC>
+__global__ void __launch_bounds__(256)
+qk_pairs_norm_k_write_vec_kernel(TA* __restrict__ proj, size_t row_len, int q_off, int k_off,
+                                 const float* __restrict__ inv_freq, int rot_dims, const float* __restrict__ q_gain,
+                                 const float* __restrict__ k_gain, int norm, float eps, const int32_t* __restrict__ tok_pos,
+                                 const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ page_table, int table_width,
+                                 TC* __restrict__ k_pages, int heads, int kv_heads, int dim, int page_size) {
+    const int lane = threadIdx.x & (RI_WAVE - 1), wave = threadIdx.x / RI_WAVE;
+    const int t = blockIdx.x;
+    const int lanes_per_head = dim / 8;                      // a power of two, at most 64
+    const int heads_at_once = RI_WAVE / lanes_per_head;
+    const int pos = tok_pos[t];
+    const int page = page_table[(size_t)tok_seq[t] * table_width + pos / page_size];
+    const int qk_heads = heads + kv_heads;
+    TA* row = proj + (size_t)t * row_len;
+    const int sub = lane / lanes_per_head, piece = lane % lanes_per_head;
+    float sn[4], cs[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int i = piece * 8 + 2 * e;                     // this pair: elements i and i + 1 of a head
+        sn[e] = 0.f;
+        cs[e] = 1.f;
+        if (i + 1 < rot_dims) sincosf((float)pos * inv_freq[i / 2], &sn[e], &cs[e]);
+    }
+    for (int h0 = wave * heads_at_once; h0 < qk_heads; h0 += 4 * heads_at_once) {
+        const int hh = h0 + sub;
+        if (hh >= qk_heads) continue;                        // lanes of a head stay together: the shuffles below are safe
+        const bool is_q = hh < heads;
+        TA* x = row + (is_q ? q_off + (size_t)hh * dim : k_off + (size_t)(hh - heads) * dim) + piece * 8;
+        float a[8];
+        Eight<TA>::load(x, a);
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float u = a[2 * e], v = a[2 * e + 1];
+            a[2 * e] = u * cs[e] - v * sn[e];
+            a[2 * e + 1] = v * cs[e] + u * sn[e];
+            ss += a[2 * e] * a[2 * e] + a[2 * e + 1] * a[2 * e + 1];
+        }
+        if (norm) {
+            for (int m = lanes_per_head / 2; m > 0; m >>= 1) ss += __shfl_xor(ss, m, RI_WAVE);
+            const float f = 1.0f / sqrtf(ss / (float)dim + eps);
+            const float* gain = is_q ? q_gain : k_gain;
+            float g[8];
+            if (gain) Eight<float>::load(gain + piece * 8, g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[e] = a[e] * f * (gain ? g[e] : 1.0f);
+        }
+        if (is_q) Eight<TA>::store(x, a);
+        else Eight<TC>::store(k_pages + (((size_t)page * kv_heads + (hh - heads)) * page_size + pos % page_size) * dim + piece * 8, a);
+    }
+}
+
 extern "C" int ri_qk_pairs_norm_kv_write(void* proj, int act_dtype, long row_len, int q_off, int k_off, int v_off,
                                          const float* inv_freq, int rot_dims, const float* q_gain, const float* k_gain,
                                          int norm, float eps, const int32_t* tok_pos, const int32_t* tok_seq,
@@ -370,6 +427,22 @@ extern "C" int ri_qk_pairs_norm_kv_write(void* proj, int act_dtype, long row_len
     // a prompt's values a page at a time, where the sizes allow it
     const bool paged_values = cu_seqlens && max_new > 1 && page_size % QT_TOKENS == 0 && seqs <= 65535 && kv_heads <= 65535 &&
                               (size_t)QT_TOKENS * (vdim + 1) * sizeof(float) <= 65536;
+    const int lph = dim / 8, unit = act_dtype == RI_BF16 ? 8 : 4;
+    if (paged_values && dim % 8 == 0 && lph <= 64 && (lph & (lph - 1)) == 0 && row_len % unit == 0 && q_off % unit == 0 &&
+        k_off % unit == 0) {
+#define RI_VEC(T)                                                                                                       \
+    qk_pairs_norm_k_write_vec_kernel<T, T><<<tokens, 256, 0, s>>>(                                                        \
+        (T*)proj, (size_t)row_len, q_off, k_off, inv_freq, rot_dims, q_gain, k_gain, norm, eps, tok_pos, tok_seq,         \
+        page_table, table_width, (T*)k_pages, heads, kv_heads, dim, page_size);                                          \
+    values_to_pages_kernel<T, T><<<dim3((max_new + QT_TOKENS - 2) / QT_TOKENS + 1, seqs, kv_heads), 256,                   \
+                                   QT_TOKENS * (vdim + 1) * sizeof(float), s>>>(                                          \
+        (const T*)proj, (size_t)row_len, (size_t)v_off, cu_seqlens, tok_pos, page_table, table_width, (T*)v_pages,        \
+        kv_heads, vdim, page_size)
+        if (act_dtype == RI_F32) { RI_VEC(float); } else { RI_VEC(bf16_t); }
+#undef RI_VEC
+        RI_LAUNCH_CHECK("qk_pairs_norm_kv_write");
+        return 0;
+    }
     // (a wavefront takes four heads of a token where the launch still has 64 wavefronts a compute unit then: below
     // that fewer, longer wavefronts do not pay)
     const int all_heads = heads + (paged_values ? 1 : 2) * kv_heads;

@@ -124,7 +124,8 @@ def paged(k, v, order, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, kv, dim, vdim, rot, lens", [(4, 2, 24, 40, 10, (35, 1, 3)), (3, 3, 64, 64, 64, (70,)),
-                                                            (2, 1, 6, 4, 0, (2, 33)), (8, 2, 128, 128, 32, (5, 1))])
+                                                            (2, 1, 6, 4, 0, (2, 33)), (8, 2, 128, 128, 32, (5, 1)),
+                                                            (2, 2, 64, 32, 12, (40, 3)), (1, 1, 512, 8, 500, (2,))])
 def test_rotation_unit_norm_and_cache_write(ops, dtype, heads, kv, dim, vdim, rot, lens):
     """q and k turn in neighbouring pairs over their first ``rot`` elements, then every head is divided by its root mean
     square; q stays in the projection's rows, k and v go to the pages.  The mixer's columns start inside a wider row
