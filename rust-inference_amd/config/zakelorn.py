@@ -99,10 +99,11 @@ class DecayAttentionSizes:
                 raise ConfigError(f"{where}: a linear-attention mixer needs {key!r}")
         heads = whole(m["heads"], where + ".heads", 1)
         dim = whole(m["dim"], where + ".dim", 1)
-        if not isinstance(m["decay"], list) or len(m["decay"]) != heads:
+        decay = m["decay"] if isinstance(m["decay"], list) else [m["decay"]] * heads     # one number: the same for every head
+        if len(decay) != heads:
             raise ConfigError(f"{where}.decay must list one decay for each of the {heads} heads")
         return cls(heads, dim, whole(m.get("vdim", dim), where + ".vdim", 1),
-                   tuple(f32(d, where + ".decay") for d in m["decay"]))
+                   tuple(f32(d, where + ".decay") for d in decay))
 
     def to_dict(self) -> dict:
         return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "decay": list(self.decay)}
