@@ -117,6 +117,17 @@ int ri_decay_step(float* out, const void* proj, int act_dtype, int row, int q_of
                   const float* head_decay, float q_scale, float* state, const int32_t* slots, int seqs, int heads, int dim,
                   int vdim, void* stream);
 
+// ri_decay_scan over prompts in chunks of 64 tokens (three launches: every chunk's own sum, the walk from chunk to
+// chunk, every chunk's outputs), where ri_decay_chunks_fit says the head sizes are taken (multiples of 4 up to 128;
+// the offsets and the row multiples of 4 too).  max_new: the most new tokens of a sequence; workspace: float32 of at
+// least ri_decay_chunks_workspace(...) floats.  The results differ from ri_decay_scan's by rounding alone.
+int ri_decay_chunks_fit(int dim, int vdim);
+long ri_decay_chunks_workspace(int seqs, int tokens, int heads, int dim, int vdim);
+int ri_decay_scan_chunked(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
+                          const float* head_decay, float q_scale, float* state, const int32_t* cu_seqlens,
+                          const int32_t* slots, int seqs, int tokens, int max_new, int heads, int dim, int vdim,
+                          float* workspace, long workspace_floats, void* stream);
+
 // The gated delta rule.  proj: [tokens, row] of act_dtype with the projections of q and k (kv_heads heads of dim each)
 // and v (heads heads of vdim) side by side from column q_off on: `channels` = 2 kv_heads dim + heads vdim columns.
 // ri_delta_prepare: per channel the causal convolution over time with taps [channels, ntaps] (last column: the

@@ -38,6 +38,7 @@ _SIGNATURES = {
     "ri_gla_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float,
                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gla_step_fits": [c_int, c_int],
+    "ri_decay_chunks_fit": [c_int, c_int],
     "ri_gla_step": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float,
                     c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gla_norm_gate": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_int, c_int, c_int,
@@ -111,6 +112,8 @@ _SIGNATURES = {
                       c_int, c_int, c_void_p],
     "ri_decay_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p,
                       c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_decay_scan_chunked": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p,
+                              c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, ctypes.c_long, c_void_p],
     "ri_embed_scaled": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p],
     "ri_branch_norm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_int, c_void_p,
                            c_int, c_int, c_void_p],
@@ -538,6 +541,33 @@ def decay_scan(proj, q_off: int, k_off: int, v_off: int, head_decay, q_scale: fl
           _dev(state, "state", torch.float32, (state.shape[0], heads, dim, vdim)),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
           seqs, tokens, heads, dim, vdim, _stream())
+    return out
+
+
+DECAY_CHUNKS_FROM = 128       # new tokens of a step's longest sequence from which the chunked form is the faster one
+
+
+def decay_chunks_fit(dim: int, vdim: int, row: int, offsets: tuple) -> bool:
+    """Whether ``decay_scan_chunked`` takes these head sizes and this place in the projection's rows (host code only)."""
+    return bool(_get("ri_decay_chunks_fit")(int(dim), int(vdim))) and row % 4 == 0 and all(o % 4 == 0 for o in offsets)
+
+
+def decay_scan_chunked(proj, q_off: int, k_off: int, v_off: int, head_decay, q_scale: float, state, cu_seqlens, slots,
+                       heads: int, dim: int, vdim: int, max_new: int) -> torch.Tensor:
+    """``decay_scan`` for prompts, in chunks of 64 tokens: with a constant decay a chunk's tokens do not wait for one
+    another (``o_i = sum_{j <= i} d^(i - j) (q_i . k_j) v_j + d^(i + 1) S0^T q_i``), so every chunk's own sum, the walk
+    from chunk to chunk and every chunk's outputs are three launches whatever the number of tokens.  float32
+    throughout; differs from ``decay_scan`` by rounding alone.  ``max_new``: the most new tokens of a sequence."""
+    tokens, row = proj.shape
+    seqs = slots.shape[0]
+    out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=proj.device)
+    need = (tokens // 64 + seqs) * heads * dim * vdim
+    work = torch.empty((need,), dtype=torch.float32, device=proj.device)
+    _call("ri_decay_scan_chunked", _dev(out, "out"), _dev(proj, "proj"), code(proj.dtype), row, int(q_off), int(k_off),
+          int(v_off), _dev(head_decay, "head_decay", torch.float32, (heads,)), float(q_scale),
+          _dev(state, "state", torch.float32, (state.shape[0], heads, dim, vdim)),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
+          seqs, tokens, int(max_new), heads, dim, vdim, _dev(work, "workspace"), need, _stream())
     return out
 
 

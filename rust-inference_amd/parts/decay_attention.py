@@ -82,6 +82,12 @@ class DecayLinearAttention(Mixer):
                 # one new token a sequence: the state in 16-byte pieces, a workgroup a sequence and head
                 o = ops.decay_step(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.slots, self.heads,
                                    self.dim, self.vdim)
+            elif (ctx.max_new >= ops.DECAY_CHUNKS_FROM and proj.dtype != torch.float32 and not self.rt.invariant
+                  and ops.decay_chunks_fit(self.dim, self.vdim, proj.shape[1], (col0, col0 + hk, col0 + 2 * hk))):
+                # a prompt: chunks of 64 tokens side by side instead of a walk token by token (float32 and the
+                # invariant mode keep the one form of the walk)
+                o = ops.decay_scan_chunked(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.cu_seqlens,
+                                           ctx.slots, self.heads, self.dim, self.vdim, ctx.max_new)
             else:
                 o = ops.decay_scan(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.cu_seqlens,
                                    ctx.slots, self.heads, self.dim, self.vdim)

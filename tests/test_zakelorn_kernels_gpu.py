@@ -465,6 +465,55 @@ def test_decay_scan_token_by_token_is_the_walk_in_blocks(ops):
         close(two, f64(one), 2e-6, "state")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H, dk, dv, lens", [(2, 64, 32, (200,)), (3, 12, 20, (64, 1, 130)), (1, 128, 128, (65, 63)),
+                                             (2, 4, 8, (129,)), (2, 100, 36, (2, 191, 128))])
+def test_decay_scan_in_chunks(ops, dtype, H, dk, dv, lens):
+    """The chunked form of the walk on states that are not zero, at slots in another order: lengths on, one below and one
+    above a chunk's edge, a head that does not decay and one that decays to nothing inside a chunk; against the plain
+    walk and against the walk token by token."""
+    assert ops.decay_chunks_fit(dk, dv, 8, (0,))
+    rng = np.random.default_rng(H * 17 + dk)
+    T = sum(lens)
+    before = 8
+    row = before + 2 * H * dk + 2 * H * dv
+    proj = rng.normal(size=(T, row))
+    if dtype == torch.bfloat16:
+        proj = bf16_round(proj)
+    decay = np.array([1.0, 0.05, 0.97][:H]).astype(np.float32).astype(np.float64)
+    slots = [2, 0, 3][:len(lens)]
+    state = (rng.normal(size=(4, H, dk, dv)) * 0.5).astype(np.float32).astype(np.float64)
+    want_state = state.copy()
+    q_at, k_at, v_at = before, before + H * dk, before + 2 * H * dk
+    want = plain_decay(proj, q_at, k_at, v_at, H, dk, dv, decay, lens, slots, want_state)
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    dev_state, walk_state = t(state), t(state)
+    args = (t(proj, dtype), q_at, k_at, v_at, t(decay), 1.0)
+    got = ops.decay_scan_chunked(*args, dev_state, t(cu, torch.int32), t(slots, torch.int32), H, dk, dv, max(lens))
+    close(got, want, 1e-5, "outputs")
+    close(dev_state, want_state, 1e-5, "state")
+    assert np.array_equal(f64(dev_state[1]), state[1])        # a slot that no sequence of the step has
+    walk = ops.decay_scan(*args, walk_state, t(cu, torch.int32), t(slots, torch.int32), H, dk, dv)
+    close(got, f64(walk), 1e-5, "chunks against the walk")
+
+
+def test_chunks_go_on_from_the_state_that_portions_left(ops):
+    """300 tokens in one step and in portions that end inside chunks, each portion from the state the one before left."""
+    rng = np.random.default_rng(8)
+    H, dk, dv, T = 2, 32, 64, 300
+    proj = rng.normal(size=(T, 2 * H * dk + H * dv))
+    decay, slot = t([1.0, 0.9]), t([1], torch.int32)
+    one = t(np.zeros((2, H, dk, dv)))
+    whole = ops.decay_scan_chunked(t(proj), 0, H * dk, 2 * H * dk, decay, 1.0, one, t([0, T], torch.int32), slot, H, dk, dv, T)
+    two, rows, at = t(np.zeros((2, H, dk, dv))), [], 0
+    for n in (130, 1, 150, 19):
+        rows.append(ops.decay_scan_chunked(t(proj[at:at + n]), 0, H * dk, 2 * H * dk, decay, 1.0, two, t([0, n], torch.int32),
+                                           slot, H, dk, dv, n))
+        at += n
+    close(torch.cat([r.cpu() for r in rows]), f64(whole), 1e-5, "portions")
+    close(two, f64(one), 1e-5, "state")
+
+
 # ---------------------------------------------------------------- the general router, the experts' closing sum
 def plain_route(z, corr, experts, identity, top, groups, keep):
     router = {"experts": experts, "identity": identity, "top": top, "groups": {"count": groups, "keep": keep}}
