@@ -9,7 +9,7 @@
 // state in the sequence's slot (a few loads and stores an element), and every chunk's outputs (all chunks side by side).
 // Only powers d^m with m >= 0 appear, so no decay is too small or too large for it.  Everything is float32: the
 // activations after silu, the powers, the scores q . k, the state and all sums; a sum runs over its tokens or channels
-// in their order.  A workgroup of 256 threads takes one (chunk, sequence, head); a thread keeps tiles of 4 x 4 results
+// in their order.  A workgroup of 512 threads takes one (chunk, sequence, head); a thread keeps tiles of 4 x 4 results
 // and reads its operands from LDS 16 bytes at a time.  Head sizes: multiples of 4 up to 128.
 #include "api.h"
 #include "common.h"
@@ -18,6 +18,8 @@
 #define DC_MAX 128               // largest key or value head
 #define DC_SLAB 32               // rows of S0 staged at a time
 #define DC_ASTRIDE (DC_TOK + 4)
+#define DC_THREADS 512           // of the workgroups that work on a chunk: two wavefronts a SIMD, one behind the other's loads
+#define DC_STAGED (DC_TOK * DC_MAX / 4 / DC_THREADS)    // most 16-byte pieces a thread stages of one operand
 
 __device__ __forceinline__ float dc_silu(float v) { return v / (1.0f + expf(-v)); }
 
@@ -38,17 +40,29 @@ __device__ __forceinline__ size_t dc_entry(int t0, int b, int c) { return (size_
 template <typename TA>
 __device__ __forceinline__ void dc_stage(float* dst, int stride, const TA* __restrict__ proj, int row, int col0, int first,
                                          int n, int width, float factor, const float* pw) {
-    const int per = width / 4;
-    for (int e = threadIdx.x; e < DC_TOK * per; e += 256) {
-        const int j = e / per, i4 = (e - j * per) * 4;
-        const float4 x = dc_ld4(proj + (size_t)(first + min(j, n - 1)) * row + col0 + i4);
-        const float f = j < n ? factor * (pw ? pw[n - 1 - j] : 1.0f) : 0.f;
-        float4 y;
-        y.x = j < n ? dc_silu(x.x) * f : 0.f;
-        y.y = j < n ? dc_silu(x.y) * f : 0.f;
-        y.z = j < n ? dc_silu(x.z) * f : 0.f;
-        y.w = j < n ? dc_silu(x.w) * f : 0.f;
-        *reinterpret_cast<float4*>(dst + j * stride + i4) = y;
+    const int per = width / 4, total = DC_TOK * per;
+    float4 x[DC_STAGED];
+    int tok[DC_STAGED], at[DC_STAGED];
+    // all of a thread's loads are asked for before the first is used
+#pragma unroll
+    for (int it = 0; it < DC_STAGED; ++it) {
+        const int e = min((int)threadIdx.x + it * DC_THREADS, total - 1);
+        tok[it] = e / per;
+        at[it] = (e - tok[it] * per) * 4;
+        x[it] = dc_ld4(proj + (size_t)(first + min(tok[it], n - 1)) * row + col0 + at[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < DC_STAGED; ++it) {
+        if ((int)threadIdx.x + it * DC_THREADS < total) {
+            const int j = tok[it];
+            const float f = j < n ? factor * (pw ? pw[n - 1 - j] : 1.0f) : 0.f;
+            float4 y;
+            y.x = j < n ? dc_silu(x[it].x) * f : 0.f;
+            y.y = j < n ? dc_silu(x[it].y) * f : 0.f;
+            y.z = j < n ? dc_silu(x[it].z) * f : 0.f;
+            y.w = j < n ? dc_silu(x[it].w) * f : 0.f;
+            *reinterpret_cast<float4*>(dst + j * stride + at[it]) = y;
+        }
     }
 }
 
@@ -59,7 +73,7 @@ __device__ __forceinline__ void dc_powers(float* pw, float d) {
 
 // U[entry, h] = sum_j d^(n - 1 - j) k_j v_j^T   [dim, vdim]
 template <typename TA>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(DC_THREADS)
 decay_chunk_sums_kernel(float* __restrict__ U, const TA* __restrict__ proj, int row, int k_off, int v_off,
                         const int32_t* __restrict__ cu_seqlens, const float* __restrict__ head_decay, int heads, int dim,
                         int vdim) {
@@ -79,19 +93,26 @@ decay_chunk_sums_kernel(float* __restrict__ U, const TA* __restrict__ proj, int 
     __syncthreads();
     float* Uc = U + (dc_entry(t0, b, c) * heads + h) * dim * vdim;
     const int tcs = vdim / 4, tiles = (dim / 4) * tcs;
-    for (int tile = threadIdx.x; tile < tiles; tile += 256) {
+    for (int tile = threadIdx.x; tile < tiles; tile += DC_THREADS) {
         const int tr = tile / tcs, tc = tile - tr * tcs;
         float acc[4][4] = {};
-        for (int j = 0; j < n; ++j) {
-            const float4 k4 = *reinterpret_cast<const float4*>(Ks + j * dim + 4 * tr);
-            const float4 v4 = *reinterpret_cast<const float4*>(Vs + j * vdim + 4 * tc);
-            const float kk[4] = {k4.x, k4.y, k4.z, k4.w};
+        for (int j0 = 0; j0 < n; j0 += 4) {                  // (the rows from n on are zeros)
+            float4 k4[4], v4[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                acc[r][0] += kk[r] * v4.x;
-                acc[r][1] += kk[r] * v4.y;
-                acc[r][2] += kk[r] * v4.z;
-                acc[r][3] += kk[r] * v4.w;
+            for (int m = 0; m < 4; ++m) {
+                k4[m] = *reinterpret_cast<const float4*>(Ks + (j0 + m) * dim + 4 * tr);
+                v4[m] = *reinterpret_cast<const float4*>(Vs + (j0 + m) * vdim + 4 * tc);
+            }
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const float kk[4] = {k4[m].x, k4[m].y, k4[m].z, k4[m].w};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    acc[r][0] += kk[r] * v4[m].x;
+                    acc[r][1] += kk[r] * v4[m].y;
+                    acc[r][2] += kk[r] * v4[m].z;
+                    acc[r][3] += kk[r] * v4[m].w;
+                }
             }
         }
 #pragma unroll
@@ -133,7 +154,7 @@ decay_chunk_carry_kernel(float* __restrict__ U, float* __restrict__ state, const
 
 // o_i = sum_{j <= i} d^(i - j) (q_i . k_j) v_j + d^(i + 1) S0^T q_i for the tokens of one chunk.
 template <typename TA>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(DC_THREADS)
 decay_chunk_out_kernel(float* __restrict__ out, const float* __restrict__ U, const TA* __restrict__ proj, int row, int q_off,
                        int k_off, int v_off, const int32_t* __restrict__ cu_seqlens, const float* __restrict__ head_decay,
                        float q_scale, int heads, int dim, int vdim) {
@@ -153,39 +174,38 @@ decay_chunk_out_kernel(float* __restrict__ out, const float* __restrict__ U, con
     dc_stage(Qs, qs, proj, row, q_off + h * dim, first, n, dim, q_scale, (const float*)nullptr);
     dc_stage(KV, qs, proj, row, k_off + h * dim, first, n, dim, 1.0f, (const float*)nullptr);
     __syncthreads();
-    {   // scores: thread (ti, tj) takes queries 4 ti .. 4 ti + 3 and keys tj, tj + 16, tj + 32, tj + 48
-        const int ti = tid / 16, tj = tid % 16;
-        float acc[4][4] = {};
+    {   // scores: thread (ti, tj) takes queries 4 ti .. 4 ti + 3 and keys tj and tj + 32
+        const int ti = tid / 32, tj = tid % 32;
+        float acc[4][2] = {};
         for (int k = 0; k < dim; k += 4) {
-            float4 q4[4], k4[4];
+            float4 q4[4], k4[2];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                q4[r] = *reinterpret_cast<const float4*>(Qs + (4 * ti + r) * qs + k);
-                k4[r] = *reinterpret_cast<const float4*>(KV + (tj + 16 * r) * qs + k);
-            }
+            for (int r = 0; r < 4; ++r) q4[r] = *reinterpret_cast<const float4*>(Qs + (4 * ti + r) * qs + k);
+#pragma unroll
+            for (int s = 0; s < 2; ++s) k4[s] = *reinterpret_cast<const float4*>(KV + (tj + 32 * s) * qs + k);
 #pragma unroll
             for (int r = 0; r < 4; ++r)
 #pragma unroll
-                for (int s = 0; s < 4; ++s)
+                for (int s = 0; s < 2; ++s)
                     acc[r][s] += q4[r].x * k4[s].x + q4[r].y * k4[s].y + q4[r].z * k4[s].z + q4[r].w * k4[s].w;
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int i = 4 * ti + r, j = tj + 16 * s;
+            for (int s = 0; s < 2; ++s) {
+                const int i = 4 * ti + r, j = tj + 32 * s;
                 As[i * DC_ASTRIDE + j] = (j <= i && i < n) ? acc[r][s] * pw[i - min(j, i)] : 0.f;
             }
     }
     __syncthreads();                                         // the keys have been read: the values take their place
     dc_stage(KV, vdim, proj, row, v_off + h * vdim, first, n, vdim, 1.0f, (const float*)nullptr);
     __syncthreads();
-    // results: tiles of 4 tokens x 4 columns, at most two a thread
+    // results: tiles of 4 tokens x 4 columns, at most one a thread
     const int tcs = vdim / 4, tiles = (DC_TOK / 4) * tcs;
-    float acc[2][4][4] = {}, from_state[2][4][4] = {};
+    float acc[1][4][4] = {}, from_state[1][4][4] = {};
 #pragma unroll
-    for (int w = 0; w < 2; ++w) {
-        const int tile = tid + w * 256;
+    for (int w = 0; w < 1; ++w) {
+        const int tile = tid + w * DC_THREADS;
         if (tile < tiles) {
             const int ti = tile / tcs, tc = tile - ti * tcs;
             for (int j = 0; j < DC_TOK; j += 4) {
@@ -213,12 +233,12 @@ decay_chunk_out_kernel(float* __restrict__ out, const float* __restrict__ U, con
     for (int k0 = 0; k0 < dim; k0 += DC_SLAB) {
         const int rows = min(DC_SLAB, dim - k0);             // a multiple of 4
         __syncthreads();                                     // the slab before has been read
-        for (int e = tid; e < rows * tcs; e += 256)
+        for (int e = tid; e < rows * tcs; e += DC_THREADS)
             *reinterpret_cast<float4*>(Ss + e * 4) = *reinterpret_cast<const float4*>(S0 + (size_t)k0 * vdim + e * 4);
         __syncthreads();
 #pragma unroll
-        for (int w = 0; w < 2; ++w) {
-            const int tile = tid + w * 256;
+        for (int w = 0; w < 1; ++w) {
+            const int tile = tid + w * DC_THREADS;
             if (tile < tiles) {
                 const int ti = tile / tcs, tc = tile - ti * tcs;
                 for (int k = 0; k < rows; k += 4) {
@@ -244,8 +264,8 @@ decay_chunk_out_kernel(float* __restrict__ out, const float* __restrict__ U, con
         }
     }
 #pragma unroll
-    for (int w = 0; w < 2; ++w) {
-        const int tile = tid + w * 256;
+    for (int w = 0; w < 1; ++w) {
+        const int tile = tid + w * DC_THREADS;
         if (tile < tiles) {
             const int ti = tile / tcs, tc = tile - ti * tcs;
 #pragma unroll
@@ -303,11 +323,11 @@ extern "C" int ri_decay_scan_chunked(float* out, const void* proj, int act_dtype
             RI_REQUIRE(e_ == hipSuccess, "decay_scan_chunked: %s", hipGetErrorString(e_));                           \
             asked = true;                                                                                            \
         }                                                                                                            \
-        decay_chunk_sums_kernel<T><<<grid, 256, lds_sums, s>>>(workspace, (const T*)proj, row, k_off, v_off, cu_seqlens, \
+        decay_chunk_sums_kernel<T><<<grid, DC_THREADS, lds_sums, s>>>(workspace, (const T*)proj, row, k_off, v_off, cu_seqlens, \
                                                                head_decay, heads, dim, vdim);                        \
         decay_chunk_carry_kernel<<<dim3((dim * vdim / 4 + 255) / 256, seqs, heads), 256, 0, s>>>(                    \
             workspace, state, cu_seqlens, slots, head_decay, heads, dim, vdim);                                      \
-        decay_chunk_out_kernel<T><<<grid, 256, lds_out, s>>>(out, workspace, (const T*)proj, row, q_off, k_off, v_off, \
+        decay_chunk_out_kernel<T><<<grid, DC_THREADS, lds_out, s>>>(out, workspace, (const T*)proj, row, q_off, k_off, v_off, \
                                                              cu_seqlens, head_decay, q_scale, heads, dim, vdim);     \
     }
     if (act_dtype == RI_F32) RI_DC_GO(float) else RI_DC_GO(bf16_t)

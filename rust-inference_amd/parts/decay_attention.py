@@ -69,6 +69,7 @@ class DecayLinearAttention(Mixer):
         self.gain = rt.place_gain(weights[self.names["norm"]])
         self.head_decay = torch.tensor(self.decay, dtype=torch.float32, device=rt.device)
         self.step_fits = ops.gla_step_fits(self.dim, self.vdim)
+        self.units = ops.compute_units()
 
     def cache_need(self):
         return StateNeed((self.heads, self.dim, self.vdim), torch.float32)
@@ -82,10 +83,11 @@ class DecayLinearAttention(Mixer):
                 # one new token a sequence: the state in 16-byte pieces, a workgroup a sequence and head
                 o = ops.decay_step(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.slots, self.heads,
                                    self.dim, self.vdim)
-            elif (ctx.max_new >= ops.DECAY_CHUNKS_FROM and proj.dtype != torch.float32 and not self.rt.invariant
+            elif (proj.dtype != torch.float32 and not self.rt.invariant
+                  and ops.decay_chunks_pay(ctx.B, proj.shape[0], ctx.max_new, self.heads, self.dim, self.vdim, self.units)
                   and ops.decay_chunks_fit(self.dim, self.vdim, proj.shape[1], (col0, col0 + hk, col0 + 2 * hk))):
-                # a prompt: chunks of 64 tokens side by side instead of a walk token by token (float32 and the
-                # invariant mode keep the one form of the walk)
+                # a long prompt of few sequences: chunks of 64 tokens side by side instead of a walk token by token
+                # (float32 and the invariant mode keep the one form of the walk)
                 o = ops.decay_scan_chunked(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.cu_seqlens,
                                            ctx.slots, self.heads, self.dim, self.vdim, ctx.max_new)
             else:

@@ -289,6 +289,35 @@ def test_keys_just_inside_and_just_outside_the_window_and_the_kept_tokens(tmp_pa
         assert rel_to_max(got["e"], want) < 1.5e-2, f"window {window}, {keep} kept, {what}"
 
 
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_prompts_in_chunks_of_the_linear_attention(folders, monkeypatch, name):
+    """bfloat16 with every step of two tokens and more sent through the chunked form of the state's walk (which small
+    models and short prompts would not take by themselves): whole prompts, portions that end inside chunks, down to two
+    tokens, and unequal batches, each going on from the state the step before left."""
+    from rust_inference_amd.kernels import ops
+    from rust_inference_amd.parts import load_model
+    monkeypatch.setattr(ops, "DECAY_CHUNKS_FORCED", True)
+    calls, chunked_form = [], ops.decay_scan_chunked
+    monkeypatch.setattr(ops, "decay_scan_chunked", lambda *a, **k: (calls.append(1), chunked_form(*a, **k))[1])
+    cfg = CONFIGS[name]
+    model = load_model(folders[name], DTYPES["bfloat16"])
+    reqs = requests_for(cfg, "c", [300, 66, 129, 2], 77)
+    batch = {rid: (toks, max(1, len(toks) - 5)) for rid, toks in reqs.items()}
+    for what, steps in (("whole", plans.whole(reqs)), ("portions", in_portions(reqs, [70, 2, 150])),
+                        ("a batch", plans.unequal_batches([batch]))):
+        against_plain(folders[name], replay(model, steps), reqs, "bfloat16", f"{name} in chunks, {what}")
+    monkeypatch.setattr(ops, "DECAY_CHUNKS_FORCED", False)
+    walked = replay(model, plans.whole(reqs))
+    monkeypatch.setattr(ops, "DECAY_CHUNKS_FORCED", True)
+    chunked = replay(model, plans.whole(reqs))
+    assert len(calls) >= 6 * len(cfg["layers"]), "the layers' linear attention did not go in chunks"
+    for rid in reqs:                                  # the two forms differ by rounding alone
+        n = settled(folders[name], reqs[rid], "bfloat16")
+        if n:
+            err = np.abs(chunked[rid][:n].astype(np.float64) - walked[rid][:n]).max() / np.abs(walked[rid][:n]).max()
+            assert err < 2e-2, f"{name}, request {rid}: chunks and walk differ by {err:.2e} of the largest logit"
+
+
 @pytest.mark.parametrize("cuts", [[300], [1] * 40 + [260], [33, 2, 265], [299, 1]])
 def test_a_state_that_does_not_decay_survives_every_cut(folders, tmp_path_factory, cuts):
     """With a decay of 1 and 0.9999 the linear attention's state keeps the first token for hundreds of steps, and the
