@@ -77,8 +77,8 @@ __global__ void __launch_bounds__(DC_THREADS)
 decay_chunk_sums_kernel(float* __restrict__ U, const TA* __restrict__ proj, int row, int k_off, int v_off,
                         const int32_t* __restrict__ cu_seqlens, const float* __restrict__ head_decay, int heads, int dim,
                         int vdim) {
-    extern __shared__ float lds[];
-    __shared__ float pw[DC_TOK + 1];
+    extern __shared__ __align__(16) float lds[];           // read 16 bytes at a time: it must start on a multiple of 16,
+    __shared__ __align__(16) float pw[DC_TOK + 4];         // so what stands before it is a multiple of 16 bytes too
     const int c = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
     const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
     const int first = t0 + c * DC_TOK;
@@ -158,8 +158,8 @@ __global__ void __launch_bounds__(DC_THREADS)
 decay_chunk_out_kernel(float* __restrict__ out, const float* __restrict__ U, const TA* __restrict__ proj, int row, int q_off,
                        int k_off, int v_off, const int32_t* __restrict__ cu_seqlens, const float* __restrict__ head_decay,
                        float q_scale, int heads, int dim, int vdim) {
-    extern __shared__ float lds[];
-    __shared__ float pw[DC_TOK + 1];
+    extern __shared__ __align__(16) float lds[];           // read 16 bytes at a time: it must start on a multiple of 16,
+    __shared__ __align__(16) float pw[DC_TOK + 4];         // so what stands before it is a multiple of 16 bytes too
     const int c = blockIdx.x, b = blockIdx.y, h = blockIdx.z, tid = threadIdx.x;
     const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
     const int first = t0 + c * DC_TOK;

@@ -229,7 +229,7 @@ def _rewrite_launches(text: str) -> str:
                    + (", " + args if args.strip() else "") + ")")
         pos = rpar + 1
     text = "".join(out)
-    return re.sub(r"extern\s+__shared__\s+(\w+)\s+(\w+)\[\];", r"\1* \2 = (\1*)emu::dyn_shared();", text)
+    return re.sub(r"extern\s+__shared__\s+(?:__align__\(\d+\)\s+)?(\w+)\s+(\w+)\[\];", r"\1* \2 = (\1*)emu::dyn_shared();", text)
 
 
 def build_emulated(out_dir: str, patches: dict | None = None) -> str:

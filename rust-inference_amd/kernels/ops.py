@@ -544,28 +544,20 @@ def decay_scan(proj, q_off: int, k_off: int, v_off: int, head_decay, q_scale: fl
     return out
 
 
-DECAY_CHUNKS_FROM = 128       # new tokens of a step's longest sequence below which the chunked form is never the faster one
+DECAY_CHUNKS_FROM = 128       # new tokens of a step's longest sequence from which the chunked form is the faster one
 DECAY_CHUNKS_FORCED = None    # True or False: every step of two tokens and more, or none, goes in chunks (tests, measurements)
 
 
-def decay_chunks_pay(seqs: int, tokens: int, max_new: int, heads: int, dim: int, vdim: int, units: int = 256) -> bool:
+def decay_chunks_pay(seqs: int, tokens: int, max_new: int, heads: int, dim: int, vdim: int) -> bool:
     """Whether ``decay_scan_chunked`` is expected to take less time than ``decay_scan`` for this step (host arithmetic
-    only).  Both estimates are fits to measurements on 256 compute units with heads of 64 x 32 to 128 x 128, 1 to 64
-    sequences and 128 to 8,192 tokens: the walk takes a token's latency (0.2 to 0.33 us) times the longest sequence,
-    and more once its workgroups (sequences x heads x sixteenths of the value head) exceed two a compute unit; the
-    chunks take a workgroup's time (60 to 200 us, by the head's size) for every 256 (chunk, head) pairs.  A long prompt
-    of few sequences goes in chunks, a batch of many prompts walks."""
+    only).  Measured on 256 compute units with heads of 64 x 32 to 128 x 128, 1 to 32 sequences and 128 to 8,192
+    tokens: the walk takes a token's latency (0.2 to 0.33 us) times the longest sequence, the chunks a workgroup's time
+    (25 to 45 us in all three launches) for as many (chunk, head) pairs as the machine holds at once; they are even at
+    128 tokens and the chunks ahead from there on, for one prompt (2,048 tokens: 67 against 672 us) and for batches of
+    prompts (32 of 1,024: 0.74 against 1.32 ms)."""
     if DECAY_CHUNKS_FORCED is not None:
         return bool(DECAY_CHUNKS_FORCED) and max_new >= 2
-    if max_new < DECAY_CHUNKS_FROM:
-        return False
-    kilo = dim * vdim / 1024.0
-    walk = (0.09 + 0.0019 * dim) * max_new * max(1.0, seqs * heads * ((vdim + 15) // 16) / (2.0 * units))
-    pairs = ((tokens + 63) // 64 + seqs - 1) * heads
-    chunks = max(50.0 + 9.5 * kilo, pairs * (0.1 + 0.043 * kilo) * 256.0 / units)
-    return chunks < 0.8 * walk
-
-
+    return max_new >= DECAY_CHUNKS_FROM
 
 
 def decay_chunks_fit(dim: int, vdim: int, row: int, offsets: tuple) -> bool:

@@ -69,7 +69,6 @@ class DecayLinearAttention(Mixer):
         self.gain = rt.place_gain(weights[self.names["norm"]])
         self.head_decay = torch.tensor(self.decay, dtype=torch.float32, device=rt.device)
         self.step_fits = ops.gla_step_fits(self.dim, self.vdim)
-        self.units = ops.compute_units()
 
     def cache_need(self):
         return StateNeed((self.heads, self.dim, self.vdim), torch.float32)
@@ -84,9 +83,9 @@ class DecayLinearAttention(Mixer):
                 o = ops.decay_step(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.slots, self.heads,
                                    self.dim, self.vdim)
             elif (proj.dtype != torch.float32 and not self.rt.invariant
-                  and ops.decay_chunks_pay(ctx.B, proj.shape[0], ctx.max_new, self.heads, self.dim, self.vdim, self.units)
+                  and ops.decay_chunks_pay(ctx.B, proj.shape[0], ctx.max_new, self.heads, self.dim, self.vdim)
                   and ops.decay_chunks_fit(self.dim, self.vdim, proj.shape[1], (col0, col0 + hk, col0 + 2 * hk))):
-                # a long prompt of few sequences: chunks of 64 tokens side by side instead of a walk token by token
+                # prompts: chunks of 64 tokens side by side instead of a walk token by token
                 # (float32 and the invariant mode keep the one form of the walk)
                 o = ops.decay_scan_chunked(proj, col0, col0 + hk, col0 + 2 * hk, self.head_decay, 1.0, store, ctx.cu_seqlens,
                                            ctx.slots, self.heads, self.dim, self.vdim, ctx.max_new)
