@@ -3,8 +3,9 @@ from .qwen3 import Qwen3Config
 from .zidepel import ZidepelConfig
 from .pisulorn import PisulornConfig
 from .zakelorn import ZakelornConfig
+from .dagezen import DagezenConfig
 from .registry import (Architecture, config_from_dict, known_architectures, load_config,
                        register_architecture, resolve_architecture)
 
-__all__ = ["ModelConfig", "Qwen3Config", "ZidepelConfig", "PisulornConfig", "ZakelornConfig", "Architecture", "read_config_json", "config_from_dict",
+__all__ = ["ModelConfig", "Qwen3Config", "ZidepelConfig", "PisulornConfig", "ZakelornConfig", "DagezenConfig", "Architecture", "read_config_json", "config_from_dict",
            "known_architectures", "load_config", "register_architecture", "resolve_architecture"]

@@ -193,6 +193,8 @@ int ri_experts_few_tokens(float* out, void* act, const void* x, const void* gu, 
 int ri_relu_squared(void* out, const void* y, int dtype, long total, void* stream);
 // out[i] = 0.5 y (1 + tanh(sqrt(2 / pi) (y + 0.044715 y^3))), in float32.
 int ri_gelu_tanh(void* out, const void* y, int dtype, long total, void* stream);
+// out[i] = 0.5 y (1 + erf(y / sqrt(2))), in float32.
+int ri_gelu_erf(void* out, const void* y, int dtype, long total, void* stream);
 
 // The same attention on the matrix cores, for bfloat16, pages of 32 tokens and head_dim 32, 64 or 128 (softcap and
 // slopes as in ri_attention; slopes NULL: no distance bias).
@@ -382,6 +384,69 @@ int ri_cache_check(void* cache);
 long ri_cache_plan_step(void* cache, const int32_t* slots, const int32_t* counts, int n, const int32_t* tokens,
                         const int32_t* want_rows, int n_want, int vocab, int width, int32_t* words, long capacity,
                         int64_t* offsets);
+
+// ---- layers whose norm sits behind the residual sum (postnorm.hip)
+// residual <- norm(alpha * residual + y + y_bias), the norm a layer norm (kind 2, with bias) or an RMS norm (kind 1); y
+// [rows, dim] or float32 [parts, rows, dim]; act: the new residual in the activations' format, or NULL.
+int ri_scaled_sum_norm(float* residual, void* act, int act_dtype, const void* y, int y_dtype, int parts,
+                       const float* y_bias, float alpha, const float* gain, const float* bias, float eps, int kind,
+                       int rows, int dim, void* stream);
+// out [rows, ff] = g sigmoid(1.702 g) (u + 1), g = min(gate + b_gate, limit), u = clamp(up + b_up, -limit, limit), for
+// gu [rows, gate | up]; the biases may be NULL.
+int ri_glu_clamped_bias(void* out, const void* gu, int dtype, const float* b_gate, const float* b_up, float limit,
+                        int rows, int ff, void* stream);
+// out [tokens, experts * ff] = dense[t, e] * act(u[t, e, :]); kind 0: exact GELU, 1: its tanh form, 2: squared ReLU;
+// dense NULL: every weight 1.
+int ri_experts_activate_plain(void* out, const void* u, int dtype, const float* dense, int dense_stride, int tokens,
+                              int experts, int ff, int kind, void* stream);
+// x <- cap * tanh(x / cap) in place.
+int ri_softcap_rows(float* x, float cap, long total, void* stream);
+
+// ---- attention over a cached latent (latent.hip)
+int ri_latent_prepare(void* proj, int act_dtype, int stride, int q_off, int kv_off, const float* gain, float eps,
+                      const float* inv_freq, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
+                      int table_width, void* k_pages, void* v_pages, int cache_dtype, int page_size, int tokens, int heads,
+                      int dim, int rot, int rank, void* stream);
+// out[t, out_off + h * out_head + 0..n) = scale * sigmoid(gates[t, g_off + h]) * x[t, x_off + h * x_head + 0..k) W_h, W
+// [heads, k, n]; the extra elements of x behind k are copied behind n; gates may be NULL.
+int ri_head_products(void* out, int out_dtype, int out_stride, int out_off, int out_head, const void* x, int x_dtype,
+                     int x_stride, int x_off, int x_head, const void* w, int w_dtype, const void* gates, int g_stride,
+                     int g_off, float scale, int tokens, int heads, int k, int n, int extra, void* stream);
+
+// ---- windowed attention whose heads talk (talking_attention.hip)
+int ri_whole_norm_kv_write(void* proj, int act_dtype, int stride, int q_off, int k_off, const float* q_gain,
+                           const float* k_gain, float eps, const int32_t* tok_pos, const int32_t* tok_seq,
+                           const int32_t* page_table, int table_width, void* k_pages, void* v_pages, int cache_dtype,
+                           int page_size, int tokens, int heads, int kv_heads, int dim, void* stream);
+int ri_talking_attention(void* out, int out_stride, int out_off, float out_scale, const void* q, int act_dtype, int q_stride,
+                         int q_off, const void* k_pages, const void* v_pages, int cache_dtype, const int32_t* tok_pos,
+                         const int32_t* tok_seq, const int32_t* page_table, int table_width, int tokens, int heads,
+                         int kv_heads, int dim, int page_size, int window, float scale, const float* r1, const float* r2,
+                         const float* talk, void* stream);
+
+// ---- time mixing (timemix.hip)
+int ri_shift_mix(void* out, int out_dtype, const float* x, const float* kept, const float* mu, int n_mix,
+                 const int32_t* tok_seq, const int32_t* cu_seqlens, const int32_t* slots, int tokens, int width, void* stream);
+int ri_shift_keep(float* kept, const float* x, const int32_t* cu_seqlens, const int32_t* slots, int seqs, int width,
+                  void* stream);
+int ri_timemix_max_dim();
+int ri_tanh_rows(void* out, int out_dtype, const float* x, long total, void* stream);
+int ri_timemix_scan(void* out, int out_stride, int out_off, float out_scale, const void* r, const void* k, const void* v,
+                    const void* g, int act_dtype, const float* z, const float* w0, const float* u, const float* gain,
+                    float eps, float* state, const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int dim,
+                    void* stream);
+
+// ---- the state-space mixer (ssd.hip)
+// update_tails 0: the convolution; 1: the tails move on by the step's tokens (call it after the convolution).
+int ri_causal_conv_silu(float* out, const void* proj, int act_dtype, int stride, int col0, const float* taps_w,
+                        const float* bias, float* tails, int taps, const int32_t* tok_seq, const int32_t* cu_seqlens,
+                        const int32_t* slots, int tokens, int seqs, int channels, int update_tails, void* stream);
+int ri_ssd_scan(float* out, const float* xbc, int channels, int b_off, int c_off, const void* proj, int act_dtype, int stride,
+                int z_off, int dt_off, const float* dt_bias, const float* a_log, const float* d_skip, float* state,
+                const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int groups, int n, int vdim,
+                void* stream);
+int ri_group_rms_norm(void* out, int out_dtype, const float* x, const float* gain, float eps, int rows, int width, int parts,
+                      void* stream);
 
 #ifdef __cplusplus
 }

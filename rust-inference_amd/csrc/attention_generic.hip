@@ -11,10 +11,10 @@
 // online softmax with running maximum m, running sum l and factor exp(m_old - m_new)
 // (the reference: src/attention.rs:117-149; its GPU form src/cuda/kernels.cu:345-405).
 //
-// Any head size from 1 to 512 (the reference asks only that it be even, and only because of its rotation:
+// Any head size from 1 to 1,024 (the reference asks only that it be even, and only because of its rotation:
 // src/models/config.rs:98-100; its own attention test runs head size 8, src/attention.rs:189-219): keys are
 // read 16 bytes at a time where a key row starts on a 16-byte boundary (head sizes that are multiples of 4
-// in float32, of 8 in bfloat16) and element by element otherwise; a thread accumulates up to two channels.
+// in float32, of 8 in bfloat16) and element by element otherwise; a thread accumulates up to four channels.
 // The value heads may have another size (v_dim) than the query and key heads.
 #include "api.h"
 #include "common.h"
@@ -42,7 +42,8 @@ template <> struct Vec<bf16_t> {
     }
 };
 
-#define ATT_MAX_HEAD_DIM (2 * ATT_TILE)
+#define ATT_ACCS 4                              // channels of a value head a thread accumulates
+#define ATT_MAX_HEAD_DIM (ATT_ACCS * ATT_TILE)
 
 template <typename TA, typename TC, bool VEC>
 __global__ void __launch_bounds__(ATT_TILE)
@@ -68,6 +69,7 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
     __syncthreads();
 
     float m = -INFINITY, l = 0.f, acc = 0.f, acc2 = 0.f;      // channels tid and tid + 256
+    float acc3 = 0.f, acc4 = 0.f;                              // and tid + 512, tid + 768 (value heads above 512)
     const int kept = min(keep_first, lo);         // keys 0..kept-1 are seen although they lie behind the window
     const int lo_tile = lo / ATT_TILE, kept_tiles = (kept + ATT_TILE - 1) / ATT_TILE;
     for (int tile = 0; tile <= qpos / ATT_TILE; ++tile) {
@@ -105,13 +107,17 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
         if (tid < v_dim) {
             acc *= corr;
             acc2 *= corr;
+            acc3 *= corr;
+            acc4 *= corr;
             const int base = tile * ATT_TILE;
             const int last = min(qpos, base + ATT_TILE - 1) - base;
-            const bool second = tid + ATT_TILE < v_dim;
+            const bool second = tid + ATT_TILE < v_dim, third = tid + 2 * ATT_TILE < v_dim, fourth = tid + 3 * ATT_TILE < v_dim;
             for (int jj = 0; jj <= last; ++jj) {
                 if (base + jj < lo && base + jj >= kept) continue;         // not seen: no weight, and no offset either
                 acc += ps[jj] * to_f32(v_pages[rowoff[jj] + (long)tid * page_size]);
                 if (second) acc2 += ps[jj] * to_f32(v_pages[rowoff[jj] + (long)(tid + ATT_TILE) * page_size]);
+                if (third) acc3 += ps[jj] * to_f32(v_pages[rowoff[jj] + (long)(tid + 2 * ATT_TILE) * page_size]);
+                if (fourth) acc4 += ps[jj] * to_f32(v_pages[rowoff[jj] + (long)(tid + 3 * ATT_TILE) * page_size]);
             }
         }
         __syncthreads();                                   // before the next tile overwrites ps and rowoff
@@ -119,6 +125,8 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
     if (sinks) l += expf(sinks[h] - m);                    // the sink: a term of the denominator alone
     if (tid < v_dim) from_f32(out + ((size_t)t * heads + h) * v_dim + tid, acc / l);
     if (tid + ATT_TILE < v_dim) from_f32(out + ((size_t)t * heads + h) * v_dim + tid + ATT_TILE, acc2 / l);
+    if (tid + 2 * ATT_TILE < v_dim) from_f32(out + ((size_t)t * heads + h) * v_dim + tid + 2 * ATT_TILE, acc3 / l);
+    if (tid + 3 * ATT_TILE < v_dim) from_f32(out + ((size_t)t * heads + h) * v_dim + tid + 3 * ATT_TILE, acc4 / l);
 }
 
 template <typename T, bool VEC>

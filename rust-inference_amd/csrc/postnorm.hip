@@ -1,0 +1,171 @@
+// Row-wise kernels of layers whose norm sits behind the residual sum, and of their feed-forwards:
+//   scaled_sum_norm:       r <- norm(alpha * r + y + y_bias): the residual itself is the norm's output (a layer norm with
+//                          gain and bias, or an RMS norm with gain); y may come as parts of a split product, added in
+//                          order, and y_bias is the bias of the product that made y; with a copy of the new r in the
+//                          activations' format, which the next sublayer's products read;
+//   glu_clamped_bias:      a = g sigmoid(1.702 g) (u + 1) with g = min(gate + b_gate, limit), u = clamp(up + b_up, -limit,
+//                          limit), for rows [gate | up];
+//   experts_activate_plain: a[t, e, :] = weight[t, e] * act(u[t, e, :]) for experts without a gate, zero for the experts a
+//                          token did not choose;
+//   softcap_rows:          x <- cap * tanh(x / cap) in place.
+//
+// The residual, the statistics, alpha and every activation are float32; a value is rounded once, when it is stored in
+// the activations' format.  One workgroup a row; a row's sums are taken in an order that the row's width alone fixes.
+#include "api.h"
+#include "common.h"
+
+#define PN_NORM_RMS 1
+#define PN_NORM_LAYER 2
+
+template <typename TY, typename TA>
+__global__ void __launch_bounds__(256)
+scaled_sum_norm_kernel(float* __restrict__ residual, TA* __restrict__ act, const TY* __restrict__ y, int parts,
+                       size_t part_stride, const float* __restrict__ y_bias, float alpha, const float* __restrict__ gain,
+                       const float* __restrict__ bias, float eps, int kind, int dim) {
+    extern __shared__ float row[];                           // dim floats
+    __shared__ float scratch[16];
+    const size_t at = (size_t)blockIdx.x * dim;
+    float sum = 0.f;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        float v = to_f32(y[at + d]);
+        for (int p = 1; p < parts; ++p) v += to_f32(y[p * part_stride + at + d]);
+        if (y_bias) v += y_bias[d];
+        v += alpha * residual[at + d];
+        row[d] = v;
+        sum += v;
+    }
+    float mean = 0.f;
+    if (kind == PN_NORM_LAYER) mean = block_sum(sum, scratch) / (float)dim;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        const float c = row[d] - mean;
+        ss += c * c;
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)dim + eps);
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        float v = (row[d] - mean) * inv * gain[d];
+        if (bias) v += bias[d];
+        residual[at + d] = v;
+        if (act) from_f32(act + at + d, v);
+    }
+}
+
+extern "C" int ri_scaled_sum_norm(float* residual, void* act, int act_dtype, const void* y, int y_dtype, int parts,
+                                  const float* y_bias, float alpha, const float* gain, const float* bias, float eps,
+                                  int kind, int rows, int dim, void* stream) {
+    RI_REQUIRE(rows > 0 && dim > 0 && parts >= 1, "scaled_sum_norm: %d rows of %d in %d parts", rows, dim, parts);
+    RI_REQUIRE(kind == PN_NORM_RMS || kind == PN_NORM_LAYER, "scaled_sum_norm: norm kind %d", kind);
+    RI_REQUIRE(gain && residual && y, "scaled_sum_norm: a gain, a residual and a branch output are needed");
+    RI_REQUIRE((size_t)dim * sizeof(float) <= 64 * 1024, "scaled_sum_norm: rows of %d exceed the kernel's 16384", dim);
+    RI_REQUIRE((y_dtype == RI_F32 || y_dtype == RI_BF16) && (act_dtype == RI_F32 || act_dtype == RI_BF16),
+               "scaled_sum_norm: dtypes %d and %d", y_dtype, act_dtype);
+    RI_REQUIRE(parts == 1 || y_dtype == RI_F32, "scaled_sum_norm: parts of a product are float32");
+    hipStream_t s = (hipStream_t)stream;
+    const size_t lds = (size_t)dim * sizeof(float), stride = (size_t)rows * dim;
+#define RI_GO(TY, TA)                                                                                                   \
+    scaled_sum_norm_kernel<TY, TA><<<rows, 256, lds, s>>>(residual, (TA*)act, (const TY*)y, parts, stride, y_bias, alpha, \
+                                                          gain, bias, eps, kind, dim)
+    if (y_dtype == RI_F32) { if (act_dtype == RI_F32) RI_GO(float, float); else RI_GO(float, bf16_t); }
+    else                   { if (act_dtype == RI_F32) RI_GO(bf16_t, float); else RI_GO(bf16_t, bf16_t); }
+#undef RI_GO
+    RI_LAUNCH_CHECK("scaled_sum_norm");
+    return 0;
+}
+
+// ------------------------------------------------------------------ the clamped gated activation with biases
+template <typename T>
+__global__ void __launch_bounds__(256)
+glu_clamped_bias_kernel(T* __restrict__ out, const T* __restrict__ gu, const float* __restrict__ b_gate,
+                        const float* __restrict__ b_up, float limit, int ff) {
+    const size_t t = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= ff) return;
+    float g = to_f32(gu[t * 2 * ff + i]), u = to_f32(gu[t * 2 * ff + ff + i]);
+    if (b_gate) g += b_gate[i];
+    if (b_up) u += b_up[i];
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    from_f32(out + t * ff + i, g / (1.f + expf(-1.702f * g)) * (u + 1.f));
+}
+
+extern "C" int ri_glu_clamped_bias(void* out, const void* gu, int dtype, const float* b_gate, const float* b_up,
+                                   float limit, int rows, int ff, void* stream) {
+    RI_REQUIRE(rows > 0, "glu_clamped_bias: %d rows", rows);
+    RI_REQUIRE(ff > 0 && limit > 0.f, "glu_clamped_bias: width %d, limit %g", ff, (double)limit);
+    RI_REQUIRE(dtype == RI_F32 || dtype == RI_BF16, "glu_clamped_bias: dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+    for (int r0 = 0; r0 < rows; r0 += 65535) {                 // the grid's second axis takes 65,535 rows
+        const int n = rows - r0 < 65535 ? rows - r0 : 65535;
+        const dim3 grid((ff + 255) / 256, n);
+        if (dtype == RI_F32)
+            glu_clamped_bias_kernel<float><<<grid, 256, 0, s>>>((float*)out + (size_t)r0 * ff, (const float*)gu + (size_t)r0 * 2 * ff,
+                                                               b_gate, b_up, limit, ff);
+        else
+            glu_clamped_bias_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out + (size_t)r0 * ff,
+                                                                (const bf16_t*)gu + (size_t)r0 * 2 * ff, b_gate, b_up, limit, ff);
+    }
+    RI_LAUNCH_CHECK("glu_clamped_bias");
+    return 0;
+}
+
+// ------------------------------------------------------------------ experts without a gate
+#define PN_ACT_GELU_ERF 0
+#define PN_ACT_GELU_TANH 1
+#define PN_ACT_RELU2 2
+
+__device__ __forceinline__ float pn_activate(float v, int kind) {
+    if (kind == PN_ACT_GELU_ERF) return 0.5f * v * (1.f + erff(v * 0.7071067811865476f));
+    if (kind == PN_ACT_GELU_TANH) return 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    const float r = fmaxf(v, 0.f);
+    return r * r;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+experts_activate_plain_kernel(T* __restrict__ out, const T* __restrict__ u, const float* __restrict__ dense,
+                              int dense_stride, int experts, int ff, int kind) {
+    const size_t t = blockIdx.y;
+    const int e = blockIdx.x;
+    const float w = dense ? dense[t * dense_stride + e] : 1.f;
+    const size_t at = (t * experts + e) * ff;
+    for (int i = threadIdx.x; i < ff; i += 256)
+        from_f32(out + at + i, w == 0.f ? 0.f : w * pn_activate(to_f32(u[at + i]), kind));
+}
+
+extern "C" int ri_experts_activate_plain(void* out, const void* u, int dtype, const float* dense, int dense_stride,
+                                         int tokens, int experts, int ff, int kind, void* stream) {
+    RI_REQUIRE(tokens > 0 && experts >= 1 && experts <= 65535 && ff >= 1, "experts_activate_plain: %d tokens, %d experts of %d",
+               tokens, experts, ff);
+    RI_REQUIRE(!dense || dense_stride >= experts, "experts_activate_plain: weight rows of %d for %d experts", dense_stride, experts);
+    RI_REQUIRE(kind >= 0 && kind <= 2, "experts_activate_plain: activation %d", kind);
+    RI_REQUIRE(dtype == RI_F32 || dtype == RI_BF16, "experts_activate_plain: dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+    for (int r0 = 0; r0 < tokens; r0 += 65535) {
+        const int n = tokens - r0 < 65535 ? tokens - r0 : 65535;
+        const dim3 grid(experts, n);
+        const size_t at = (size_t)r0 * experts * ff;
+        const float* d = dense ? dense + (size_t)r0 * dense_stride : nullptr;
+        if (dtype == RI_F32)
+            experts_activate_plain_kernel<float><<<grid, 256, 0, s>>>((float*)out + at, (const float*)u + at, d, dense_stride,
+                                                                     experts, ff, kind);
+        else
+            experts_activate_plain_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out + at, (const bf16_t*)u + at, d, dense_stride,
+                                                                      experts, ff, kind);
+    }
+    RI_LAUNCH_CHECK("experts_activate_plain");
+    return 0;
+}
+
+// ------------------------------------------------------------------ a cap on the logits
+__global__ void softcap_kernel(float* __restrict__ x, float cap, long total) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < total) x[e] = cap * tanhf(x[e] / cap);
+}
+
+extern "C" int ri_softcap_rows(float* x, float cap, long total, void* stream) {
+    RI_REQUIRE(total > 0 && cap > 0.f, "softcap_rows: %ld elements, cap %g", total, (double)cap);
+    RI_REQUIRE((total + 255) / 256 <= 2147483647L, "softcap_rows: %ld elements exceed one launch", total);
+    softcap_kernel<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, cap, total);
+    RI_LAUNCH_CHECK("softcap_rows");
+    return 0;
+}

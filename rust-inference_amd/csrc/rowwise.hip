@@ -316,7 +316,7 @@ extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int in
 // ------------------------------------------------------------------ activations of a dense feed-forward
 // out[i] = act(y[i]), taken in float32.  ACT_RELU2: max(y, 0)^2.  ACT_GELU_TANH: the tanh form of GELU,
 // 0.5 y (1 + tanh(sqrt(2 / pi) (y + 0.044715 y^3))).
-enum { ACT_RELU2 = 0, ACT_GELU_TANH = 1 };
+enum { ACT_RELU2 = 0, ACT_GELU_TANH = 1, ACT_GELU_ERF = 2 };
 
 template <int ACT>
 __device__ __forceinline__ float activate(float v) {
@@ -324,6 +324,7 @@ __device__ __forceinline__ float activate(float v) {
         const float r = fmaxf(v, 0.f);
         return r * r;
     }
+    if (ACT == ACT_GELU_ERF) return 0.5f * v * (1.f + erff(v * 0.7071067811865476f));      // the exact form
     return 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
 }
 
@@ -370,6 +371,10 @@ extern "C" int ri_relu_squared(void* out, const void* y, int dtype, long total, 
 
 extern "C" int ri_gelu_tanh(void* out, const void* y, int dtype, long total, void* stream) {
     return launch_activation<ACT_GELU_TANH>("gelu_tanh", out, y, dtype, total, stream);
+}
+
+extern "C" int ri_gelu_erf(void* out, const void* y, int dtype, long total, void* stream) {
+    return launch_activation<ACT_GELU_ERF>("gelu_erf", out, y, dtype, total, stream);
 }
 
 // ------------------------------------------------------------------ bias

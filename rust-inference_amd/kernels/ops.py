@@ -45,6 +45,7 @@ _SIGNATURES = {
                          c_void_p],
     "ri_relu_squared": [c_void_p, c_void_p, c_int, ctypes.c_long, c_void_p],
     "ri_gelu_tanh": [c_void_p, c_void_p, c_int, ctypes.c_long, c_void_p],
+    "ri_gelu_erf": [c_void_p, c_void_p, c_int, ctypes.c_long, c_void_p],
     "ri_delta_prepare": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_delta_max_dim": [],
@@ -126,6 +127,31 @@ _SIGNATURES = {
     "ri_experts_activate_strided": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ri_experts_finish": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int,
                           c_void_p],
+    "ri_scaled_sum_norm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_float,
+                           c_int, c_int, c_int, c_void_p],
+    "ri_glu_clamped_bias": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_int, c_int, c_void_p],
+    "ri_experts_activate_plain": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_softcap_rows": [c_void_p, c_float, ctypes.c_long, c_void_p],
+    "ri_latent_prepare": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_head_products": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
+                         c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_whole_norm_kv_write": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
+                               c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_talking_attention": [c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
+                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
+                             c_void_p, c_void_p],
+    "ri_shift_mix": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ri_shift_keep": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ri_timemix_max_dim": [],
+    "ri_tanh_rows": [c_void_p, c_int, c_void_p, ctypes.c_long, c_void_p],
+    "ri_timemix_scan": [c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                        c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ri_causal_conv_silu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                            c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_ssd_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                    c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_group_rms_norm": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_void_p],
 }
 
 _fn = {}
@@ -645,7 +671,15 @@ def gelu_tanh(y: torch.Tensor) -> torch.Tensor:
     return out
 
 
-ACTIVATIONS = {"relu2": relu_squared, "gelu_tanh": gelu_tanh}      # what a dense feed-forward may name
+def gelu_erf(y: torch.Tensor) -> torch.Tensor:
+    """``0.5 y (1 + erf(y / sqrt(2)))`` elementwise, taken in float32."""
+    out = torch.empty(y.shape, dtype=y.dtype, device=y.device)
+    if y.numel():
+        _call("ri_gelu_erf", _dev(out, "out"), _dev(y, "y"), code(y.dtype), y.numel(), _stream())
+    return out
+
+
+ACTIVATIONS = {"relu2": relu_squared, "gelu_tanh": gelu_tanh, "gelu_erf": gelu_erf}      # what a dense feed-forward may name
 
 DELTA_MAX_DIM = 256
 DELTA_MAX_TAPS = 16
@@ -1214,3 +1248,228 @@ def linked_product(x, w: torch.Tensor, n: int, packed: bool, out_dtype=torch.bfl
           _dev(next_gain, "next_gain", torch.float32, (n,)), _dev(xg.data if tiled_out else xg, "xg"), _dev(ssq, "ssq"),
           *layout, _stream())
     return NormedLater(xg, ssq, next_eps, n)
+
+
+# ---------------------------------------------------------------- layers whose norm sits behind the residual sum
+def scaled_sum_norm(residual: torch.Tensor, y: torch.Tensor, y_bias, alpha: float, gain, bias, eps: float, norm_kind: int,
+                    act_dtype=None):
+    """``residual <- norm(alpha * residual + y + y_bias)`` in place (float32), the norm a layer norm (``NORM_LAYER``, with
+    ``bias``) or an RMS norm (``NORM_RMS``) with ``gain``; ``y`` is ``[T, dim]`` or float32 ``[parts, T, dim]`` (added in
+    order), ``y_bias`` a float32 row or None.  With ``act_dtype`` the new residual is also returned in that format."""
+    rows, dim = residual.shape
+    parts = y.shape[0] if y.dim() == 3 else 1
+    if tuple(y.shape[-2:]) != (rows, dim):
+        raise ShapeError(f"a branch output of {list(y.shape)} for a residual of {list(residual.shape)}")
+    act = torch.empty((rows, dim), dtype=act_dtype, device=residual.device) if act_dtype is not None else None
+    _call("ri_scaled_sum_norm", _dev(residual, "residual", torch.float32), _opt(act, "act"), code(act_dtype or torch.float32),
+          _dev(y, "y"), code(y.dtype), parts, _opt(y_bias, "y_bias", torch.float32, (dim,)), float(alpha),
+          _dev(gain, "gain", torch.float32, (dim,)), _opt(bias, "bias", torch.float32, (dim,)), float(eps), int(norm_kind),
+          rows, dim, _stream())
+    return act
+
+
+def glu_clamped_bias(gu: torch.Tensor, b_gate, b_up, limit: float) -> torch.Tensor:
+    """``g sigmoid(1.702 g) (u + 1)`` with ``g = min(gate + b_gate, limit)``, ``u = clamp(up + b_up, -limit, limit)`` for rows
+    ``gu [T, gate | up]``; the biases are float32 rows or None."""
+    rows, two = gu.shape
+    ff = two // 2
+    if two != 2 * ff:
+        raise ShapeError(f"gate|up rows of {two} elements")
+    out = torch.empty((rows, ff), dtype=gu.dtype, device=gu.device)
+    _call("ri_glu_clamped_bias", _dev(out, "out"), _dev(gu, "gu"), code(gu.dtype), _opt(b_gate, "b_gate", torch.float32, (ff,)),
+          _opt(b_up, "b_up", torch.float32, (ff,)), float(limit), rows, ff, _stream())
+    return out
+
+
+PLAIN_ACTIVATIONS = {"gelu_erf": 0, "gelu_tanh": 1, "relu2": 2}      # what experts without a gate may name
+
+
+def experts_activate_plain(u: torch.Tensor, dense, ff: int, activation: str) -> torch.Tensor:
+    """``dense[t, e] * act(u[t, e, :])`` for ``u [T, E * ff]``, zero for the experts a token did not choose; ``dense`` None:
+    every weight 1."""
+    tokens, wide = u.shape
+    experts = wide // ff
+    if wide != experts * ff or (dense is not None and (dense.shape[0] != tokens or dense.shape[1] < experts)):
+        raise ShapeError(f"up rows are {list(u.shape)} for experts of {ff}, weights {None if dense is None else list(dense.shape)}")
+    out = torch.empty_like(u)
+    _call("ri_experts_activate_plain", _dev(out, "out"), _dev(u, "u"), code(u.dtype), _opt(dense, "dense", torch.float32),
+          dense.shape[1] if dense is not None else experts, tokens, experts, ff, PLAIN_ACTIVATIONS[activation], _stream())
+    return out
+
+
+def softcap_rows(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place (float32); returns ``x``."""
+    if x.numel():
+        _call("ri_softcap_rows", _dev(x, "x", torch.float32), float(cap), x.numel(), _stream())
+    return x
+
+
+# ---------------------------------------------------------------- attention over a cached latent
+GENERIC_MAX_HEAD_DIM = 1024      # what the general attention kernel alone takes
+
+
+def latent_prepare(proj, q_off: int, kv_off: int, gain, eps: float, inv_freq, tok_pos, tok_seq, page_table, k_pages, v_pages,
+                   heads: int, dim: int, rot: int, rank: int) -> None:
+    """In rows ``proj [T, ...]``: the latent (``rank`` columns from ``kv_off``) is RMS-normed with ``gain`` and written, with
+    the rotated ``rot`` columns behind it, as the token's key row ``[rank + rot]`` of one key/value head, and alone as its
+    value row; the last ``rot`` elements of every query head (``heads`` of ``dim + rot`` from ``q_off``) are rotated in place."""
+    tokens, stride = proj.shape
+    if tuple(k_pages.shape[1:]) != (1, v_pages.shape[3], rank + rot) or tuple(v_pages.shape[1:3]) != (1, rank):
+        raise ShapeError(f"latent_prepare: key pages {list(k_pages.shape)}, value pages {list(v_pages.shape)} for a latent of "
+                         f"{rank} + {rot}")
+    _call("ri_latent_prepare", _dev(proj, "proj"), code(proj.dtype), stride, int(q_off), int(kv_off),
+          _dev(gain, "gain", torch.float32, (rank,)), float(eps), _opt(inv_freq, "inv_freq", torch.float32, (rot // 2,)),
+          _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1], _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
+          code(k_pages.dtype), k_pages.shape[2], tokens, heads, dim, rot, rank, _stream())
+
+
+def head_products(x, x_off: int, x_head: int, w, heads: int, k: int, n: int, extra: int = 0, out=None, out_off: int = 0,
+                  out_head: int | None = None, gates=None, g_off: int = 0, scale: float = 1.0, out_dtype=None):
+    """``out[t, out_off + h * out_head + (0..n)] = scale * sigmoid(gates[t, g_off + h]) * x[t, x_off + h * x_head + (0..k)] @ w[h]``
+    for a stack of matrices ``w [heads, k, n]``; the ``extra`` elements of ``x`` behind ``k`` are copied behind ``n`` (times
+    the same factors).  ``out`` None: a new tensor ``[T, heads * (n + extra)]`` of ``out_dtype`` (default: ``x``'s)."""
+    tokens = x.shape[0]
+    if tuple(w.shape) != (heads, k, n):
+        raise ShapeError(f"head_products: matrices {list(w.shape)} for {heads} heads of {k} x {n}")
+    if out is None:
+        out_head = n + extra
+        out = torch.empty((tokens, heads * out_head), dtype=out_dtype or x.dtype, device=x.device)
+    if out.shape[0] != tokens or (gates is not None and (gates.shape[0] != tokens or gates.dtype != x.dtype)):
+        raise ShapeError(f"head_products: out {list(out.shape)}, x {list(x.shape)}")
+    _call("ri_head_products", _dev(out, "out"), code(out.dtype), out.shape[1], int(out_off), int(out_head), _dev(x, "x"),
+          code(x.dtype), x.shape[1], int(x_off), int(x_head), _dev(w, "w"), code(w.dtype), _opt(gates, "gates"),
+          gates.shape[1] if gates is not None else 0, int(g_off), float(scale), tokens, heads, k, n, int(extra), _stream())
+    return out
+
+
+# ---------------------------------------------------------------- windowed attention whose heads talk
+def whole_norm_kv_write(proj, q_off: int, k_off: int, q_gain, k_gain, eps: float, tok_pos, tok_seq, page_table, k_pages,
+                        v_pages, heads: int, kv_heads: int, dim: int) -> None:
+    """q (``heads * dim`` columns from ``q_off``) and k (``kv_heads * dim`` from ``k_off``) of every row are RMS-normed over
+    the whole projection with a gain an element; q stays in place, the normed k goes to the key pages and k as projected
+    to the value pages."""
+    tokens, stride = proj.shape
+    if tuple(k_pages.shape[1:]) != (kv_heads, v_pages.shape[3], dim) or tuple(v_pages.shape[1:3]) != (kv_heads, dim):
+        raise ShapeError(f"whole_norm_kv_write: key pages {list(k_pages.shape)}, value pages {list(v_pages.shape)}")
+    _call("ri_whole_norm_kv_write", _dev(proj, "proj"), code(proj.dtype), stride, int(q_off), int(k_off),
+          _dev(q_gain, "q_gain", torch.float32, (heads * dim,)), _dev(k_gain, "k_gain", torch.float32, (kv_heads * dim,)),
+          float(eps), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1], _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
+          code(k_pages.dtype), k_pages.shape[2], tokens, heads, kv_heads, dim, _stream())
+
+
+def talking_attention(out, out_off: int, out_scale: float, proj, q_off: int, k_pages, v_pages, tok_pos, tok_seq, page_table,
+                      heads: int, kv_heads: int, dim: int, window: int | None, scale: float, r1, r2, talk) -> None:
+    """Windowed attention of every new token over its sequence's pages with the distance bias ``r1_h ln(1 + r2_h (i - j))``
+    taken off the scores and the heads' weights mixed by ``talk [heads, heads]`` after the softmax; the heads' results,
+    times ``out_scale``, go to the columns ``out_off ..`` of ``out``.  ``r1``/``r2`` and ``talk`` may be None."""
+    tokens = proj.shape[0]
+    if out.shape[0] != tokens or out.dtype != proj.dtype:
+        raise ShapeError(f"talking_attention: out {list(out.shape)} {out.dtype} for rows {list(proj.shape)} {proj.dtype}")
+    _call("ri_talking_attention", _dev(out, "out"), out.shape[1], int(out_off), float(out_scale), _dev(proj, "proj"),
+          code(proj.dtype), proj.shape[1], int(q_off), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), code(k_pages.dtype),
+          _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1], tokens, heads, kv_heads, dim, k_pages.shape[2],
+          int(window or 0), float(scale), _opt(r1, "r1", torch.float32, (heads,)), _opt(r2, "r2", torch.float32, (heads,)),
+          _opt(talk, "talk", torch.float32, (heads, heads)), _stream())
+
+
+# ---------------------------------------------------------------- time mixing
+def timemix_max_dim() -> int:
+    return _get("ri_timemix_max_dim")()
+
+
+def shift_mix(x32, kept, mu, tok_seq, cu_seqlens, slots, out_dtype) -> torch.Tensor:
+    """``[n, T, width]``: for every mixing vector ``mu[s]`` the rows ``h + (h' - h) * mu[s]``, ``h'`` the row before (the
+    sequence's kept row ``kept[slot]`` for the first token of the step)."""
+    tokens, width = x32.shape
+    n = mu.shape[0]
+    out = torch.empty((n, tokens, width), dtype=out_dtype, device=x32.device)
+    _call("ri_shift_mix", _dev(out, "out"), code(out_dtype), _dev(x32, "x", torch.float32), _dev(kept, "kept", torch.float32),
+          _dev(mu, "mu", torch.float32, (n, width)), n, _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32), _dev(slots, "slots", torch.int32), tokens, width, _stream())
+    return out
+
+
+def tanh_rows(x: torch.Tensor, out_dtype) -> torch.Tensor:
+    """``tanh(x)`` of float32 ``x``, taken in float32 and written as ``out_dtype``."""
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    if x.numel():
+        _call("ri_tanh_rows", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.float32), x.numel(), _stream())
+    return out
+
+
+def shift_keep(kept, x32, cu_seqlens, slots) -> None:
+    """Every sequence's last row of the step becomes its kept row."""
+    seqs = slots.shape[0]
+    _call("ri_shift_keep", _dev(kept, "kept", torch.float32), _dev(x32, "x", torch.float32),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32), seqs, x32.shape[1], _stream())
+
+
+def timemix_scan(out, out_off: int, out_scale: float, r, k, v, g, z, w0, u, gain, eps: float, state, cu_seqlens, slots,
+                 heads: int, dim: int) -> None:
+    """The walk of the time mixing over every sequence's new tokens on ``state [slots, heads, dim, dim]`` (float32, in
+    place); ``r, k, v, g [T, heads * dim]``, ``z`` float32 the decay's pre-activation without its bias ``w0``; the normed and
+    gated heads, times ``out_scale``, go to the columns ``out_off ..`` of ``out``."""
+    tokens, width = r.shape
+    seqs = slots.shape[0]
+    for name, t in (("k", k), ("v", v), ("g", g)):
+        if tuple(t.shape) != (tokens, width) or t.dtype != r.dtype:
+            raise ShapeError(f"timemix_scan: {name} is {list(t.shape)} {t.dtype}, r {list(r.shape)} {r.dtype}")
+    if width != heads * dim or tuple(state.shape[1:]) != (heads, dim, dim) or out.shape[0] != tokens or out.dtype != r.dtype:
+        raise ShapeError(f"timemix_scan: rows of {width}, state {list(state.shape)}, out {list(out.shape)}")
+    _call("ri_timemix_scan", _dev(out, "out"), out.shape[1], int(out_off), float(out_scale), _dev(r, "r"), _dev(k, "k"),
+          _dev(v, "v"), _dev(g, "g"), code(r.dtype), _dev(z, "z", torch.float32, (tokens, width)),
+          _dev(w0, "w0", torch.float32, (width,)), _dev(u, "u", torch.float32, (width,)),
+          _dev(gain, "gain", torch.float32, (width,)), float(eps), _dev(state, "state", torch.float32),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32), seqs, heads, dim, _stream())
+
+
+# ---------------------------------------------------------------- the state-space mixer
+SSD_MAX_TAPS = 16
+
+
+def causal_conv_silu(proj, col0: int, channels: int, taps_w, bias, tails, tok_seq, cu_seqlens, slots) -> torch.Tensor:
+    """float32 ``[T, channels]``: ``silu`` of every channel's causal convolution (``taps_w [channels, taps]``, the last
+    column the current token's) over the columns ``col0 ..`` of ``proj``, the inputs before a step from ``tails [slots, taps -
+    1, channels]``; then the tails are moved on by the step's tokens."""
+    tokens = proj.shape[0]
+    seqs, taps = slots.shape[0], taps_w.shape[1]
+    if tuple(taps_w.shape) != (channels, taps) or (taps > 1 and tuple(tails.shape[1:]) != (taps - 1, channels)):
+        raise ShapeError(f"causal_conv_silu: taps {list(taps_w.shape)}, tails {list(tails.shape)} for {channels} channels")
+    out = torch.empty((tokens, channels), dtype=torch.float32, device=proj.device)
+    for update in (0, 1):
+        _call("ri_causal_conv_silu", _dev(out, "out"), _dev(proj, "proj"), code(proj.dtype), proj.shape[1], int(col0),
+              _dev(taps_w, "taps", torch.float32), _opt(bias, "bias", torch.float32, (channels,)),
+              _opt(tails if taps > 1 else None, "tails", torch.float32), taps, _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+              _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32), tokens, seqs,
+              channels, update, _stream())
+    return out
+
+
+def ssd_scan(xbc, b_off: int, c_off: int, proj, z_off: int, dt_off: int, dt_bias, a_log, d_skip, state, cu_seqlens, slots,
+             heads: int, groups: int, n: int, vdim: int) -> torch.Tensor:
+    """float32 ``[T, heads * vdim]``: the walk ``S <- exp(-exp(A_log) dt) S + dt B x^T``, ``y = S^T C + D x`` over every
+    sequence's new tokens on ``state [slots, heads, n, vdim]`` (float32, in place), times ``silu(z)``; x, B and C are
+    columns of ``xbc`` (float32), z and the raw step sizes columns of ``proj``."""
+    tokens, channels = xbc.shape
+    seqs = slots.shape[0]
+    if tuple(state.shape[1:]) != (heads, n, vdim) or proj.shape[0] != tokens:
+        raise ShapeError(f"ssd_scan: state {list(state.shape)} for {heads} heads of {n} x {vdim}")
+    out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=xbc.device)
+    _call("ri_ssd_scan", _dev(out, "out"), _dev(xbc, "xbc", torch.float32), channels, int(b_off), int(c_off), _dev(proj, "proj"),
+          code(proj.dtype), proj.shape[1], int(z_off), int(dt_off), _opt(dt_bias, "dt_bias", torch.float32, (heads,)),
+          _dev(a_log, "a_log", torch.float32, (heads,)), _opt(d_skip, "d_skip", torch.float32, (heads,)),
+          _dev(state, "state", torch.float32), _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)),
+          _dev(slots, "slots", torch.int32), seqs, heads, groups, n, vdim, _stream())
+    return out
+
+
+def group_rms_norm(x, gain, eps: float, parts: int, out_dtype) -> torch.Tensor:
+    """Rows of float32 ``x [T, width]`` in ``parts`` equal parts, each divided by its root mean square, times ``gain``."""
+    rows, width = x.shape
+    out = torch.empty((rows, width), dtype=out_dtype, device=x.device)
+    _call("ri_group_rms_norm", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.float32),
+          _opt(gain, "gain", torch.float32, (width,)), float(eps), rows, width, int(parts), _stream())
+    return out

@@ -1,5 +1,5 @@
-from . import (attention, block, decay_attention, delta, experts, feed_forward, gla, norm, parallel, position, streams,
-               qwen3, zidepel, pisulorn, zakelorn)  # noqa: F401  (registers the parts)
+from . import (attention, block, decay_attention, delta, experts, feed_forward, gla, latent, norm, parallel, position,
+               postnorm, ssd, streams, talking, timemix, qwen3, zidepel, pisulorn, zakelorn, dagezen)  # noqa: F401  (registers the parts)
 from .base import Embedding, FeedForward, Head, Mixer, Norm, Part, PositionEncoding
 from .block import PreNormBlock, ResidualStream
 from .context import StepContext

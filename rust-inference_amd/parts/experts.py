@@ -37,6 +37,9 @@ class RoutedExperts(FeedForward):
     ``keep`` best groups can be chosen.  ``identity=n``: the router has ``n`` more outputs after the experts', which
     stand for experts that hand the token's own row on (times the weight) and have no tensors; they are scored,
     grouped and chosen like the others.  ``limit=None``: an expert is ``W_down (silu(W_gate h) (W_up h))``.
+    ``gated=False, activation=...``: an expert is ``W_down act(W_up h)`` (``<prefix>e<i>.up`` and ``.down`` alone), ``act`` one of
+    ``ops.PLAIN_ACTIVATIONS``.  ``router_bias=True``: the logits are ``W_router h + b`` (``<prefix>router.b``) and there is no
+    correction; with ``scores="softmax"`` and ``normalize=True`` the weights are then the softmax over the chosen logits alone.
     ``shared=ff``: one more expert of that width and form, ``<prefix>shared.gate`` / ``.up`` / ``.down``, runs for
     every token and is added times ``sigmoid(W_sg h)``, one number a token (``<prefix>shared.sg [1, hidden]``; its row
     rides as the last row of the router's matrix).
@@ -44,8 +47,14 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, hidden: int, inter: int, experts: int, top: int, limit: float | None, prefix: str,
                  scores: str = "sigmoid", normalize: bool = True, groups: tuple | None = None, identity: int = 0,
-                 shared: int | None = None):
+                 shared: int | None = None, gated: bool = True, activation: str | None = None, router_bias: bool = False):
         self.outs = experts + int(identity)
+        self.gated, self.activation, self.router_bias = bool(gated), activation, bool(router_bias)
+        if not self.gated:
+            if activation not in ops.PLAIN_ACTIVATIONS:
+                raise ConfigError(f"experts without a gate name one of {', '.join(sorted(ops.PLAIN_ACTIVATIONS))}, not {activation!r}")
+            if identity or shared is not None or limit is not None:
+                raise ConfigError("experts without a gate take no limit, no identity experts and no shared expert")
         if not 1 <= top <= self.outs <= ops.EXPERTS_MAX or experts < 1:
             raise ConfigError(f"the {top} best of {experts} experts and {identity} identity experts: the router takes up to "
                               f"{ops.EXPERTS_MAX} outputs")
@@ -65,14 +74,18 @@ class RoutedExperts(FeedForward):
     def tensors(self):
         p, t = self.prefix, {}
         t[p + "router"] = TensorSpec((self.outs, self.hidden), MATRIX)
-        t[p + "correction"] = TensorSpec((self.outs,), BIAS)
+        if self.router_bias:
+            t[p + "router.b"] = TensorSpec((self.outs,), BIAS)
+        else:
+            t[p + "correction"] = TensorSpec((self.outs,), BIAS)
         if self.shared is not None:
             t[p + "shared.gate"] = TensorSpec((self.shared, self.hidden), MATRIX)
             t[p + "shared.up"] = TensorSpec((self.shared, self.hidden), MATRIX)
             t[p + "shared.down"] = TensorSpec((self.hidden, self.shared), MATRIX)
             t[p + "shared.sg"] = TensorSpec((1, self.hidden), MATRIX)
         for e in range(self.experts):
-            t[f"{p}e{e}.gate"] = TensorSpec((self.inter, self.hidden), MATRIX)
+            if self.gated:
+                t[f"{p}e{e}.gate"] = TensorSpec((self.inter, self.hidden), MATRIX)
             t[f"{p}e{e}.up"] = TensorSpec((self.inter, self.hidden), MATRIX)
             t[f"{p}e{e}.down"] = TensorSpec((self.hidden, self.inter), MATRIX)
         return t
@@ -87,10 +100,15 @@ class RoutedExperts(FeedForward):
                                        swiglu=True)
             self.w_shared_down = rt.pack(rt.place_matrix(weights[p + "shared.down"]), parts_ok=True)
         self.w_router = rt.pack(rt.place_matrix(router))
-        self.correction = rt.place_gain(weights[p + "correction"])
+        if self.router_bias:
+            # a bias of the router's product: it moves the logits themselves, so choice and weights both see it
+            self.z_bias = rt.place_gain(weights[p + "router.b"])
+            self.correction = torch.zeros_like(self.z_bias)
+        else:
+            self.z_bias, self.correction = None, rt.place_gain(weights[p + "correction"])
         rows = []
         for e in range(self.experts):
-            rows += [weights[f"{p}e{e}.gate"], weights[f"{p}e{e}.up"]]
+            rows += [weights[f"{p}e{e}.gate"], weights[f"{p}e{e}.up"]] if self.gated else [weights[f"{p}e{e}.up"]]
         self.w_gate_up = rt.pack(rt.place_matrix(torch.cat(rows, 0)), always=True)
         down = torch.cat([weights[f"{p}e{e}.down"] for e in range(self.experts)], 1)
         self.w_down = rt.pack(rt.place_matrix(down), parts_ok=True)
@@ -106,6 +124,8 @@ class RoutedExperts(FeedForward):
         rt = self.rt
         with profiler.section(profiler.MLP):
             z = ops.as_rows(rt.linear_packed(x, self.w_router, out_dtype=torch.float32))
+            if self.z_bias is not None:
+                z = ops.add_bias(z, self.z_bias)
             extra = None
             if self.simple:
                 ids, weights, dense = ops.experts_route(z, self.correction, self.top)
@@ -116,8 +136,9 @@ class RoutedExperts(FeedForward):
             tokens = z.shape[0]
             routed = (rt.dtype == torch.bfloat16 and not rt.invariant and self.top < self.experts
                       and self.hidden % 8 == 0 and self.inter % 8 == 0)
+            few = routed and self.gated          # the kernel that reads the chosen experts' rows alone knows gated experts
             own = self.identity > 0                   # whether the identity experts' share is still to be added
-            if routed and tokens * self.top < self.experts:
+            if few and tokens * self.top < self.experts:
                 y, own = ops.experts_few_tokens(rt.normed_now(x), self.w_gate_up.w, self.w_down.w, ids, weights, self.inter,
                                                 self.limit), False
             elif (routed and tokens >= self.SORTED_MIN_TOKENS and not ctx.is_decode
@@ -125,7 +146,8 @@ class RoutedExperts(FeedForward):
                 y, own = self.forward_sorted(rt.normed_now(x), ids, weights), False
             else:
                 gu = ops.as_rows(rt.linear_packed(x, self.w_gate_up))
-                a = ops.experts_activate(gu, dense, self.inter, self.limit)
+                a = (ops.experts_activate(gu, dense, self.inter, self.limit) if self.gated
+                     else ops.experts_activate_plain(gu, dense, self.inter, self.activation))
                 # float32 into the residual (or in parts that the stream's next read adds)
                 y = rt.linear_packed(a, self.w_down, out_dtype=torch.float32, parts_ok=True)
             if not own and self.shared is None:
@@ -140,6 +162,7 @@ class RoutedExperts(FeedForward):
         """A prompt: every expert's tokens as rows side by side, two library products an expert, the weighted sum in
         float32.  The host reads how many rows every expert has (one wait a layer), which a captured step could not."""
         ff = self.inter
+        rows_each = 2 * ff if self.gated else ff
         dest, offsets = ops.experts_sort(ids, self.outs)
         rows = ops.experts_gather(x, dest, self.top)
         y = torch.empty_like(rows)
@@ -147,8 +170,9 @@ class RoutedExperts(FeedForward):
         for e in range(self.experts):
             a, b = starts[e], starts[e + 1]
             if b > a:
-                gu = torch.mm(rows[a:b], self.w_gate_up.w[e * 2 * ff:(e + 1) * 2 * ff].t())
-                act = ops.experts_activate(gu, None, ff, self.limit)
+                gu = torch.mm(rows[a:b], self.w_gate_up.w[e * rows_each:(e + 1) * rows_each].t())
+                act = (ops.experts_activate(gu, None, ff, self.limit) if self.gated
+                       else ops.experts_activate_plain(gu, None, ff, self.activation))
                 torch.mm(act, self.w_down.w[:, e * ff:(e + 1) * ff].t(), out=y[a:b])
         if self.identity and starts[self.outs] > starts[self.experts]:
             y[starts[self.experts]:] = rows[starts[self.experts]:]        # identity experts: the token's own row

@@ -6,7 +6,7 @@ import torch
 from .. import profiler
 from ..errors import ConfigError
 from ..kernels import ops
-from ..weights.loader import MATRIX, TensorSpec
+from ..weights.loader import BIAS, MATRIX, TensorSpec
 from .base import FeedForward
 from .registry import register_part
 
@@ -90,6 +90,49 @@ class DenseFF(FeedForward):
         with profiler.section(profiler.MLP):
             a = ops.ACTIVATIONS[self.activation](ops.as_rows(rt.linear_packed(x, self.w_up)))
             # float32 into the residual (or in parts that the stream's next read adds): the sum is never rounded to 16 bits
+            return rt.linear_packed(a, self.w_down, out_dtype=torch.float32, parts_ok=True)
+
+
+@register_part("feed_forward", "glu_clamped")
+class ClampedGatedFF(FeedForward):
+    """``down(g sigmoid(1.702 g) (u + 1))`` with ``g = min(gate(x), limit)`` and ``u = clamp(up(x), -limit, limit)``; with
+    ``biases`` every product has one (``<name>.b``).  Gate and up are one product with the row-concatenated weight; their
+    biases, the clamps and the activation are one kernel; the bias of the last product is offered to the residual
+    stream (``out_bias``), which adds it where it adds the product.  ``names`` gives the checkpoint names of ``gate``,
+    ``up`` and ``down`` where they are not ``<prefix>gate`` and so on."""
+
+    def __init__(self, hidden: int, inter: int, limit: float, prefix: str, biases: bool = True, names: dict | None = None):
+        if not limit > 0:
+            raise ConfigError(f"the limit {limit} of a clamped feed-forward must be positive")
+        self.hidden, self.inter, self.limit, self.prefix, self.biases = hidden, inter, float(limit), prefix, bool(biases)
+        self.names = {"gate": prefix + "gate", "up": prefix + "up", "down": prefix + "down"}
+        self.names.update(names or {})
+        self.out_bias = None
+
+    def tensors(self):
+        n = self.names
+        t = {n["gate"]: TensorSpec((self.inter, self.hidden), MATRIX), n["up"]: TensorSpec((self.inter, self.hidden), MATRIX),
+             n["down"]: TensorSpec((self.hidden, self.inter), MATRIX)}
+        if self.biases:
+            t.update({n["gate"] + ".b": TensorSpec((self.inter,), BIAS), n["up"] + ".b": TensorSpec((self.inter,), BIAS),
+                      n["down"] + ".b": TensorSpec((self.hidden,), BIAS)})
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        n = self.names
+        self.w_gate_up = rt.pack(rt.place_matrix(torch.cat([weights[n["gate"]], weights[n["up"]]], 0)), always=True)
+        self.w_down = rt.pack(rt.place_matrix(weights[n["down"]]), parts_ok=True)
+        self.b_gate = rt.place_gain(weights[n["gate"] + ".b"]) if self.biases else None
+        self.b_up = rt.place_gain(weights[n["up"] + ".b"]) if self.biases else None
+        self.out_bias = rt.place_gain(weights[n["down"] + ".b"]) if self.biases else None
+
+    def forward(self, x, ctx):
+        rt = self.rt
+        with profiler.section(profiler.MLP):
+            gu = ops.as_rows(rt.linear_packed(x, self.w_gate_up))
+            a = ops.glu_clamped_bias(gu, self.b_gate, self.b_up, self.limit)
+            # float32 into the residual (or in parts that the stream's next read adds); the last bias rides as out_bias
             return rt.linear_packed(a, self.w_down, out_dtype=torch.float32, parts_ok=True)
 
 

@@ -88,12 +88,13 @@ class PositionedEmbedding(Embedding):
 
 @register_part("head", "linear")
 class OutputHead(Head):
-    """``logits = x W^T`` in float32, no scaling or cap.  The matrix is the embedding
+    """``logits = x W^T`` in float32, no scaling; with ``softcap`` the logits are then capped, ``c tanh(logits / c)``.  The matrix is the embedding
     table when the configuration ties them or the checkpoint has no tensor of this
     name (the reference: src/models/qwen3.rs:167-171, :286)."""
 
-    def __init__(self, vocab: int, dim: int, name: str, tied: bool):
+    def __init__(self, vocab: int, dim: int, name: str, tied: bool, softcap: float | None = None):
         self.vocab, self.dim, self.name, self.tied = vocab, dim, name, tied
+        self.softcap = float(softcap) if softcap else None      # logits <- cap * tanh(logits / cap), in float32
 
     def tensors(self):
         return {self.name: TensorSpec((self.vocab, self.dim), MATRIX, optional=True)}
@@ -153,6 +154,10 @@ class OutputHead(Head):
     PAIRED_MAX_ROWS = 8
 
     def forward(self, x):
+        logits = self.uncapped(x)
+        return ops.softcap_rows(logits, self.softcap) if self.softcap is not None else logits
+
+    def uncapped(self, x):
         rows = x.shape[0]
         if self.rt.invariant:
             return self.rt.linear_packed(x, self._packed_copy(), out_dtype=torch.float32)

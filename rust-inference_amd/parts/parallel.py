@@ -21,7 +21,16 @@ class ParallelMixers(Mixer):
     product (``in_matrix``, ``core``, ``out_matrix``: the attention of the third family, the linear attention with a
     fixed decay) share both products: one product with all members' input rows, the members' cores write their heads,
     times their constant, side by side into one row, and one product with the output matrices side by side along K
-    adds the members up in its float32 sum.  Other members run whole, and their float32 results are added."""
+    adds the members up in its float32 sum.  Members that make their own input products but can write their finished heads
+    into a row of another's (``run_into`` and ``out_matrix``: an attention whose heads talk, time mixing, whose five
+    projections each read a mix of their own) share the output product alone.  Other members run whole, and their float32
+    results are added.
+
+    A member that keeps several things per sequence (a tuple of needs) gets its stores as a tuple; the layer's run names
+    the members' entries one after the other.  A member that sets ``wants_residual`` also gets the float32 residual the
+    layer hands over (``residual=``)."""
+
+    wants_residual = True
 
     def __init__(self, mixers: tuple, scales: tuple):
         if len(mixers) < 1 or len(mixers) != len(scales):
@@ -30,6 +39,8 @@ class ParallelMixers(Mixer):
         self.scales = tuple(float(s) for s in scales)
         self.fused = all(hasattr(m, "core") and hasattr(m, "in_matrix") and hasattr(m, "out_matrix") and
                          (getattr(m, "paired", True)) for m in self.members)
+        # members that write their heads into one row for one output product, each after input products of its own
+        self.shares_out = not self.fused and all(hasattr(m, "run_into") and hasattr(m, "out_matrix") for m in self.members)
 
     def tensors(self):
         t = {}
@@ -39,6 +50,16 @@ class ParallelMixers(Mixer):
 
     def bind(self, weights, rt):
         self.rt = rt
+        if self.shares_out:
+            for m in self.members:
+                m.bind(weights, rt, alone=False)
+            self.w_out = rt.pack(rt.place_matrix(torch.cat([m.out_matrix(weights) for m in self.members], 1)), parts_ok=True)
+            self.out_at, b = [], 0
+            for m in self.members:
+                self.out_at.append(b)
+                b += m.out_width
+            self.out_width = b
+            return
         if not self.fused:
             for m in self.members:
                 m.bind(weights, rt)
@@ -55,16 +76,42 @@ class ParallelMixers(Mixer):
         self.out_width = b
 
     def cache_need(self):
-        return tuple(m.cache_need() for m in self.members)
+        needs = []
+        for m in self.members:
+            need = m.cache_need()
+            needs += list(need) if isinstance(need, (tuple, list)) else [need]
+        return tuple(needs)
 
-    def forward(self, x, ctx, stores, page_tables):
+    def _per_member(self, stores, page_tables):
+        """The stores and page tables of a run, dealt out to the members: one each, or a tuple for a member with several needs."""
+        out, at = [], 0
+        for m in self.members:
+            need = m.cache_need()
+            if isinstance(need, (tuple, list)):
+                out.append((tuple(stores[at:at + len(need)]), tuple(page_tables[at:at + len(need)])))
+                at += len(need)
+            else:
+                out.append((stores[at], page_tables[at]))
+                at += 1
+        return out
+
+    def forward(self, x, ctx, stores, page_tables, residual=None):
         rt = self.rt
         if not isinstance(stores, tuple):
             stores, page_tables = (stores,), (page_tables,)
+        dealt = self._per_member(stores, page_tables)
+        extra = lambda m: {"residual": residual} if getattr(m, "wants_residual", False) else {}
+        if self.shares_out:
+            rows = x.shape[0]
+            heads = torch.empty((rows, self.out_width), dtype=rt.dtype, device=rt.device)
+            for m, scale, (store, table), b in zip(self.members, self.scales, dealt, self.out_at):
+                m.run_into(x, ctx, store, table, heads, b, scale, **extra(m))
+            with profiler.section(profiler.OUT_PROJECTION):
+                return rt.linear_packed(heads, self.w_out, out_dtype=torch.float32, parts_ok=True)
         if not self.fused:
             total = None
-            for m, scale, store, table in zip(self.members, self.scales, stores, page_tables):
-                y = m.forward(x, ctx, store, table)
+            for m, scale, (store, table) in zip(self.members, self.scales, dealt):
+                y = m.forward(x, ctx, store, table, **extra(m))
                 if isinstance(y, tuple):
                     raise ConfigError("a mixer side by side with others hands back its result, not a link to a norm")
                 if y.dim() == 3:
@@ -75,7 +122,7 @@ class ParallelMixers(Mixer):
         with profiler.section(profiler.QKV_PROJECTION):
             proj = ops.as_rows(rt.linear_packed(x, self.w_in))
         heads = torch.empty((proj.shape[0], self.out_width), dtype=proj.dtype, device=proj.device)
-        for m, scale, store, table, a, b in zip(self.members, self.scales, stores, page_tables, self.in_at, self.out_at):
+        for m, scale, (store, table), a, b in zip(self.members, self.scales, dealt, self.in_at, self.out_at):
             m.core(proj, a, ctx, store, table, heads, b, scale)
         with profiler.section(profiler.OUT_PROJECTION):
             return rt.linear_packed(heads, self.w_out, out_dtype=torch.float32, parts_ok=True)
