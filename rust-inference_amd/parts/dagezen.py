@@ -64,7 +64,7 @@ def dagezen_spec(cfg: DagezenConfig) -> ModelSpec:
             parts["feed_forward"] = _feed_forward(cfg, layer.mlp, p + "mlp.")
             parts["feed_forward_norm"] = _norm(cfg, p + "norm2")
         layers.append(LayerSpec("norm_after_sum", parts))
-        schedule.append(Run(layer=i, cache=tuple(range(entry, entry + kept))))
+        schedule.append(Run(layer=i, cache=entry if kept == 1 else tuple(range(entry, entry + kept))))
         entry += kept
     return ModelSpec(
         architecture=cfg.ARCHITECTURE,

@@ -144,7 +144,7 @@ def test_latent_attention_through_every_cut(ops, heads, dim, rot, vdim, rank):
          "g": rng.standard_normal((heads, width)) / 6, "o": np.eye(heads * vdim)}
     inv_freq = t(100.0 ** (-2.0 * np.arange(rot // 2) / rot))
     w_uk = t(w["uk"].reshape(heads, dim, rank))
-    w_uv = t(w["uv"].reshape(heads, vdim, rank).transpose(0, 2, 1))
+    w_uv = t(np.ascontiguousarray(w["uv"].reshape(heads, vdim, rank).transpose(0, 2, 1)))
     lengths = [43, 43]
     h = [rng.standard_normal((n, width)) for n in lengths]
     steps = Steps(lengths, [0, 1], rng)
