@@ -2,7 +2,7 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--model 8b|0.6b|1.7b|4b|14b|32b]
-    python bench.py --design zidepel|pisulorn|zakelorn [--size 0.6b|8b] [--layers L]      # another workload: see design_comparison below
+    python bench.py --design zidepel|pisulorn|zakelorn|dagezen [--size 0.6b|8b] [--layers L]      # another workload: see design_comparison below
 
 The default run has the layer sizes of Qwen3-8B with random weights
 (N(0, 0.02), norm gains 1 + N(0, 0.1), seed 2), a batch of 8 and prompts of 2,048 tokens in a
@@ -246,6 +246,28 @@ def zakelorn_like(q, layers, vocab, context):
             "layers": [{"type": "parallel", "mixer": mixer, "mlp": (dense, moe, None, moe)[i % 4]} for i in range(layers)]}
 
 
+def dagezen_like(q, layers, vocab, context):
+    """A Dagezen configuration with the layer sizes of a Qwen3 one: the same width; of every four layers the first is
+    attention over a cached latent of four head sizes with half a head size of rotated elements (Qwen3's heads and head
+    size) and a dense clamped feed-forward half again as wide as Qwen3's; the second and the fourth are a windowed
+    attention whose heads talk (Qwen3's heads and key heads, a window of 1,024 keys) beside time mixing with a quarter
+    as many heads of the same size, with eight experts of half Qwen3's width of which a token uses two; the third is a
+    state-space mixer with Qwen3's heads and head size, a state of one head size, its key heads as groups, four taps,
+    and no feed-forward."""
+    d, h, g, dh, ff = q["hidden_size"], q["num_attention_heads"], q["num_key_value_heads"], q["head_dim"], q["intermediate_size"]
+    lat = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": ff * 3 // 2, "limit": 7.0},
+           "mixer": {"heads": h, "dim": dh, "rot_dim": dh // 2, "vdim": dh, "kv_rank": 4 * dh, "scale": (dh + dh // 2) ** -0.5,
+                     "rot": {"dims": dh // 2, "base": 1e6}}}
+    moe = {"kind": "moe", "expert": {"ff": ff // 2}, "router": {"experts": 8, "top": 2}}
+    par = {"type": "parallel", "mlp": moe,
+           "mixer": {"left": {"heads": h, "kv_heads": g, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "mask": {"size": 1024}},
+                     "right": {"heads": max(1, h // 4), "dim": dh, "rank": 64}, "left_scale": 0.7, "right_scale": 0.7}}
+    ssm = {"type": "mamba2", "mlp": None,
+           "mixer": {"heads": h, "vdim": dh, "state": dh, "groups": g, "conv": 4, "norm_groups": g}}
+    return {"architecture": "Dagezen", "vocab": vocab, "width": d, "norm": {"eps": 1e-5}, "postln_alpha": 1.5, "logit_softcap": 30.0,
+            "layers": [(lat, par, ssm, par)[i % 4] for i in range(layers)]}
+
+
 def design_comparison(args) -> int:
     """`--design zidepel`, `--design pisulorn` or `--design zakelorn`: prefill and decode of a model of that design beside the Qwen3 model
     of the same layer sizes (and, for Pisulorn, beside the Zidepel model of those sizes, the design closest to it)
@@ -253,6 +275,28 @@ def design_comparison(args) -> int:
     the output matrix are what is timed).  One JSON line; the default workload and its line are not touched."""
     sizes = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B}
     layers, vocab, context = args.layers or 8, 32768, args.context
+    if args.design == "dagezen":
+        out = {"metric": "prefill and decode of the Dagezen design beside Zakelorn and Qwen3 at equal layer sizes", "unit": "tok/s",
+               "n_gpus": 1, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids", "layers": layers,
+               "vocab": vocab, "steps": args.steps, "warmup": args.warmup, "sizes": {}}
+        for size in ([args.size] if args.size else ["0.6b", "8b"]):
+            q = dict(sizes[size], num_hidden_layers=layers, vocab_size=vocab, max_position_embeddings=context,
+                     tie_word_embeddings=False)
+            trio = {}
+            for name, cfg in (("qwen3", q), ("zakelorn", zakelorn_like(q, layers, vocab, context)),
+                              ("dagezen", dagezen_like(q, layers, vocab, context))):
+                if args.only and name != args.only:
+                    continue
+                b = ShapeBench(f"{name} at Qwen3-{size} layer sizes", cfg, vocab, 11, context, not args.no_graphs)
+                trio[name] = b.measure(args.prompt, (1, 8, 32), args.steps, args.warmup)
+                b.close()
+            out["sizes"][size] = trio
+        first = out["sizes"][next(iter(out["sizes"]))]
+        out["value"], out["higher_is_better"] = first["dagezen"]["decode_b8"]["tok_s"], True
+        if "zakelorn" in first:
+            out["vs_zakelorn_decode_b8"] = round(first["dagezen"]["decode_b8"]["tok_s"] / first["zakelorn"]["decode_b8"]["tok_s"], 3)
+        print(json.dumps(out))
+        return 0
     if args.design == "zakelorn":
         out = {"metric": "prefill and decode of the Zakelorn design beside Pisulorn and Qwen3 at equal layer sizes", "unit": "tok/s",
                "n_gpus": 1, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids", "layers": layers,
@@ -325,9 +369,10 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the other models")
     ap.add_argument("--no-other-models", action="store_true", help="skip the Qwen3-0.6B and Qwen3-32B points")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel of a decode step from the host")
-    ap.add_argument("--design", choices=["zidepel", "pisulorn", "zakelorn"], default=None,
+    ap.add_argument("--design", choices=["zidepel", "pisulorn", "zakelorn", "dagezen"], default=None,
                     help="another workload: this design beside Qwen3 at equal layer sizes (prefill, decode at batch 1, 8, 32)")
     ap.add_argument("--size", choices=["0.6b", "8b"], default=None, help="with --design: one of the two layer sizes only")
+    ap.add_argument("--only", default=None, help="with --design dagezen: one of the models only (qwen3, zakelorn, dagezen)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this library is single-GPU, --gpus {args.gpus} is not run")
