@@ -418,11 +418,14 @@ int ri_whole_norm_kv_write(void* proj, int act_dtype, int stride, int q_off, int
                            const float* k_gain, float eps, const int32_t* tok_pos, const int32_t* tok_seq,
                            const int32_t* page_table, int table_width, void* k_pages, void* v_pages, int cache_dtype,
                            int page_size, int tokens, int heads, int kv_heads, int dim, void* stream);
-int ri_talking_attention(void* out, int out_stride, int out_off, float out_scale, const void* q, int act_dtype, int q_stride,
-                         int q_off, const void* k_pages, const void* v_pages, int cache_dtype, const int32_t* tok_pos,
-                         const int32_t* tok_seq, const int32_t* page_table, int table_width, int tokens, int heads,
-                         int kv_heads, int dim, int page_size, int window, float scale, const float* r1, const float* r2,
-                         const float* talk, void* stream);
+// shares > 1: out is float32 [shares][tokens][out_stride] partial sums for the caller to add; stats: float32 workspace
+// [tokens][heads][2].
+int ri_talking_attention_shares(int tokens, int longest);
+int ri_talking_attention(void* out, int out_dtype, int out_stride, int out_off, float out_scale, int shares, float* stats,
+                         const void* q, int act_dtype, int q_stride, int q_off, const void* k_pages, const void* v_pages,
+                         int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
+                         int table_width, int tokens, int heads, int kv_heads, int dim, int page_size, int window, float scale,
+                         const float* r1, const float* r2, const float* talk, void* stream);
 
 // ---- time mixing (timemix.hip)
 int ri_shift_mix(void* out, int out_dtype, const float* x, const float* kept, const float* mu, int n_mix,
@@ -435,6 +438,12 @@ int ri_timemix_scan(void* out, int out_stride, int out_off, float out_scale, con
                     const void* g, int act_dtype, const float* z, const float* w0, const float* u, const float* gain,
                     float eps, float* state, const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int dim,
                     void* stream);
+// The same walk with a thread a column of the state (heads of up to 128); o: float32 workspace [tokens, heads * dim].
+int ri_timemix_scan_cols_fits(int dim);
+int ri_timemix_scan_cols(void* out, int out_stride, int out_off, float out_scale, float* o, const void* r, const void* k,
+                         const void* v, const void* g, int act_dtype, const float* z, const float* w0, const float* u,
+                         const float* gain, float eps, float* state, const int32_t* cu_seqlens, const int32_t* slots, int tokens,
+                         int seqs, int heads, int dim, void* stream);
 
 // ---- the state-space mixer (ssd.hip)
 // update_tails 0: the convolution; 1: the tails move on by the step's tokens (call it after the convolution).
@@ -445,6 +454,12 @@ int ri_ssd_scan(float* out, const float* xbc, int channels, int b_off, int c_off
                 int z_off, int dt_off, const float* dt_bias, const float* a_log, const float* d_skip, float* state,
                 const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int groups, int n, int vdim,
                 void* stream);
+// The same walk with a thread a column of the state, for states of up to 128 rows.
+int ri_ssd_scan_cols_fits(int n, int vdim);
+int ri_ssd_scan_cols(float* out, const float* xbc, int channels, int b_off, int c_off, const void* proj, int act_dtype, int stride,
+                     int z_off, int dt_off, const float* dt_bias, const float* a_log, const float* d_skip, float* state,
+                     const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int groups, int n, int vdim,
+                     void* stream);
 int ri_group_rms_norm(void* out, int out_dtype, const float* x, const float* gain, float eps, int rows, int width, int parts,
                       void* stream);
 

@@ -112,6 +112,39 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
             const int base = tile * ATT_TILE;
             const int last = min(qpos, base + ATT_TILE - 1) - base;
             const bool second = tid + ATT_TILE < v_dim, third = tid + 2 * ATT_TILE < v_dim, fourth = tid + 3 * ATT_TILE < v_dim;
+            if (VEC && page_size % 8 == 0) {
+                // eight neighbouring keys of a channel lie side by side in a value page: one 16-byte load (two in
+                // float32) instead of eight elements; a key that is not seen has the weight 0
+                for (int j0 = 0; j0 <= last; j0 += 8) {
+                    const int a = base + j0, b = min(a + 7, qpos);
+                    if (b < lo && a >= kept) continue;                         // none of the eight is seen
+                    const TC* vp = v_pages + ((long)table[a / page_size] * kv_heads + kvh) * page_size * (long)v_dim +
+                                   a % page_size + (long)tid * page_size;
+                    float vv[8];
+                    Vec<TC>::load(vp, vv);
+                    if (Vec<TC>::N == 4) Vec<TC>::load(vp + 4, vv + 4);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc += ps[j0 + e] * vv[e];
+                    if (second) {
+                        Vec<TC>::load(vp + (long)ATT_TILE * page_size, vv);
+                        if (Vec<TC>::N == 4) Vec<TC>::load(vp + (long)ATT_TILE * page_size + 4, vv + 4);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) acc2 += ps[j0 + e] * vv[e];
+                    }
+                    if (third) {
+                        Vec<TC>::load(vp + 2L * ATT_TILE * page_size, vv);
+                        if (Vec<TC>::N == 4) Vec<TC>::load(vp + 2L * ATT_TILE * page_size + 4, vv + 4);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) acc3 += ps[j0 + e] * vv[e];
+                    }
+                    if (fourth) {
+                        Vec<TC>::load(vp + 3L * ATT_TILE * page_size, vv);
+                        if (Vec<TC>::N == 4) Vec<TC>::load(vp + 3L * ATT_TILE * page_size + 4, vv + 4);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) acc4 += ps[j0 + e] * vv[e];
+                    }
+                }
+            } else
             for (int jj = 0; jj <= last; ++jj) {
                 if (base + jj < lo && base + jj >= kept) continue;         // not seen: no weight, and no offset either
                 acc += ps[jj] * to_f32(v_pages[rowoff[jj] + (long)tid * page_size]);
@@ -160,7 +193,7 @@ extern "C" int ri_attention_kept(void* out, const void* q, int act_dtype, int q_
     hipStream_t s = (hipStream_t)stream;
     // a key row starts on a 16-byte boundary when the head size is a multiple of 4 (float32) or 8 (bfloat16):
     // the pools themselves are 256-byte aligned allocations
-    const bool vec = head_dim % (act_dtype == RI_F32 ? 4 : 8) == 0 && (uintptr_t)k_pages % 16 == 0;
+    const bool vec = head_dim % (act_dtype == RI_F32 ? 4 : 8) == 0 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0;
 #define RI_ATT_GO(T, V) launch_attention<T, V>(out, q, q_stride, k_pages, v_pages, tok_pos, tok_seq, page_table, \
                                                table_width, tokens, heads, kv_heads, head_dim, v_dim, page_size, window, scale, \
                                                softcap, slopes, window > 0 ? keep_first : 0, sinks, s)

@@ -189,3 +189,152 @@ extern "C" int ri_timemix_scan(void* out, int out_stride, int out_off, float out
     RI_LAUNCH_CHECK("timemix_scan");
     return 0;
 }
+
+// ------------------------------------------------------------------ the walk, a thread a column
+// Heads of up to 128: a thread holds a whole column of the state in registers, so a token's sum over the rows needs no
+// other thread, and a workgroup is one wavefront on 64 columns of one (sequence, head).  Tokens are staged in LDS in
+// blocks of TM_BLOCK (r, k, the decay, v), the next block's loads asked for before the block in work is computed.  The
+// heads' results are written as they are, float32; the norm over a head and the gate are heads_norm_gate's.
+#define TM_BLOCK 8
+
+template <typename TA, int ROWS>
+__global__ void __launch_bounds__(64)
+timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, const TA* __restrict__ k, const TA* __restrict__ v,
+                         const float* __restrict__ z, const float* __restrict__ w0, const float* __restrict__ u,
+                         float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
+                         int heads, int dim) {
+    __shared__ __attribute__((aligned(16))) float rs[2][TM_BLOCK][ROWS];
+    __shared__ __attribute__((aligned(16))) float ks[2][TM_BLOCK][ROWS];
+    __shared__ __attribute__((aligned(16))) float ws[2][TM_BLOCK][ROWS];
+    __shared__ __attribute__((aligned(16))) float us[ROWS];
+    __shared__ float vs[2][TM_BLOCK][64];
+    const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int c = blockIdx.z * 64 + lane;
+    const bool has_col = c < dim;
+    const int cc = has_col ? c : dim - 1;                     // a column pulled back inside the head: loads are issued anyway
+    const int width = heads * dim;
+    float* sp = state + (((size_t)slots[seq] * heads + h) * dim) * dim + cc;
+    float st[ROWS];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) st[i] = i < dim ? sp[(size_t)i * dim] : 0.f;
+    for (int i = lane; i < ROWS; i += 64) us[i] = i < dim ? u[h * dim + i] : 0.f;
+    const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
+    constexpr int PER = (TM_BLOCK * ROWS + 63) / 64;          // elements of each of r, k and the decay that a lane stages
+
+    float pre_r[PER], pre_k[PER], pre_w[PER], pre_v[TM_BLOCK];
+    auto fetch = [&](int tb) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = lane + i * 64;
+            const int row = e % ROWS, tt = e / ROWS;
+            const bool in = row < dim && tt < TM_BLOCK;
+            const size_t at = (size_t)min(tb + tt, t1 - 1) * width + (size_t)h * dim + (in ? row : 0);
+            pre_r[i] = in ? to_f32(r[at]) : 0.f;
+            pre_k[i] = in ? to_f32(k[at]) : 0.f;
+            pre_w[i] = in ? z[at] + w0[h * dim + row] : 0.f;
+        }
+#pragma unroll
+        for (int tt = 0; tt < TM_BLOCK; ++tt) pre_v[tt] = to_f32(v[(size_t)min(tb + tt, t1 - 1) * width + (size_t)h * dim + cc]);
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = lane + i * 64;
+            const int row = e % ROWS, tt = e / ROWS;
+            if (tt < TM_BLOCK) {
+                rs[buf][tt][row] = pre_r[i];
+                ks[buf][tt][row] = pre_k[i];
+                ws[buf][tt][row] = expf(-expf(pre_w[i]));
+            }
+        }
+#pragma unroll
+        for (int tt = 0; tt < TM_BLOCK; ++tt) vs[buf][tt][lane] = pre_v[tt];
+    };
+    if (t0 < t1) {
+        fetch(t0);
+        stage(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int tb = t0; tb < t1; tb += TM_BLOCK, buf ^= 1) {
+        const bool more = tb + TM_BLOCK < t1;
+        if (more) fetch(tb + TM_BLOCK);
+        const int count = min(TM_BLOCK, t1 - tb);
+        for (int tt = 0; tt < count; ++tt) {
+            const float vc = vs[buf][tt][lane];
+            float o = 0.f;
+#pragma unroll
+            for (int i = 0; i < ROWS; i += 4) {
+                const float4 r4 = *reinterpret_cast<const float4*>(&rs[buf][tt][i]);
+                const float4 k4 = *reinterpret_cast<const float4*>(&ks[buf][tt][i]);
+                const float4 w4 = *reinterpret_cast<const float4*>(&ws[buf][tt][i]);
+                const float4 u4 = *reinterpret_cast<const float4*>(&us[i]);
+                float kv = k4.x * vc;
+                o += (st[i] + u4.x * kv) * r4.x;             st[i] = w4.x * st[i] + kv;
+                kv = k4.y * vc;
+                o += (st[i + 1] + u4.y * kv) * r4.y;         st[i + 1] = w4.y * st[i + 1] + kv;
+                kv = k4.z * vc;
+                o += (st[i + 2] + u4.z * kv) * r4.z;         st[i + 2] = w4.z * st[i + 2] + kv;
+                kv = k4.w * vc;
+                o += (st[i + 3] + u4.w * kv) * r4.w;         st[i + 3] = w4.w * st[i + 3] + kv;
+            }
+            if (has_col) out[(size_t)(tb + tt) * width + (size_t)h * dim + c] = o;
+        }
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+    }
+    if (has_col) {
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i)
+            if (i < dim) sp[(size_t)i * dim] = st[i];
+    }
+}
+
+// out[t, out_off + h * dim + c] = scale * o[t, h, c] / sqrt(mean_c(o[t, h, :]^2) + eps) * gain[h * dim + c] * silu(g[t, h * dim + c]).
+template <typename TA>
+__global__ void __launch_bounds__(64)
+heads_norm_gate_kernel(TA* __restrict__ out, int out_stride, int out_off, float scale, const float* __restrict__ o,
+                       const float* __restrict__ gain, const TA* __restrict__ g, float eps, int heads, int dim) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    const size_t at = ((size_t)t * heads + h) * dim;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 64) ss += o[at + d] * o[at + d];
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+    for (int d = threadIdx.x; d < dim; d += 64) {
+        const float gate = to_f32(g[at + d]);
+        from_f32(out + (size_t)t * out_stride + out_off + (size_t)h * dim + d,
+                 o[at + d] * inv * gain[h * dim + d] * (gate / (1.f + expf(-gate))) * scale);
+    }
+}
+
+extern "C" int ri_timemix_scan_cols_fits(int dim) { return dim >= 1 && dim <= 128; }
+
+extern "C" int ri_timemix_scan_cols(void* out, int out_stride, int out_off, float out_scale, float* o, const void* r,
+                                    const void* k, const void* v, const void* g, int act_dtype, const float* z, const float* w0,
+                                    const float* u, const float* gain, float eps, float* state, const int32_t* cu_seqlens,
+                                    const int32_t* slots, int tokens, int seqs, int heads, int dim, void* stream) {
+    RI_REQUIRE(tokens > 0 && seqs > 0 && heads > 0 && heads <= 65535 && ri_timemix_scan_cols_fits(dim),
+               "timemix_scan_cols: %d tokens of %d sequences, %d heads of %d", tokens, seqs, heads, dim);
+    RI_REQUIRE(out_off >= 0 && out_off + heads * dim <= out_stride, "timemix_scan_cols: column %d of rows of %d", out_off, out_stride);
+    RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "timemix_scan_cols: dtype %d", act_dtype);
+    const dim3 grid(seqs, heads, (dim + 63) / 64);
+    hipStream_t s = (hipStream_t)stream;
+#define RI_GO(TA, ROWS)                                                                                                 \
+    timemix_scan_cols_kernel<TA, ROWS><<<grid, 64, 0, s>>>(o, (const TA*)r, (const TA*)k, (const TA*)v, z, w0, u, state, \
+                                                           cu_seqlens, slots, heads, dim)
+#define RI_BY_ROWS(TA)                                                                                                  \
+    if (dim <= 16) RI_GO(TA, 16); else if (dim <= 32) RI_GO(TA, 32); else if (dim <= 64) RI_GO(TA, 64); else RI_GO(TA, 128)
+    if (act_dtype == RI_F32) {
+        RI_BY_ROWS(float);
+        heads_norm_gate_kernel<float><<<dim3(tokens, heads), 64, 0, s>>>((float*)out, out_stride, out_off, out_scale, o, gain,
+                                                                        (const float*)g, eps, heads, dim);
+    } else {
+        RI_BY_ROWS(bf16_t);
+        heads_norm_gate_kernel<bf16_t><<<dim3(tokens, heads), 64, 0, s>>>((bf16_t*)out, out_stride, out_off, out_scale, o, gain,
+                                                                         (const bf16_t*)g, eps, heads, dim);
+    }
+#undef RI_BY_ROWS
+#undef RI_GO
+    RI_LAUNCH_CHECK("timemix_scan_cols");
+    return 0;
+}

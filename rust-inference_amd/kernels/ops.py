@@ -138,19 +138,27 @@ _SIGNATURES = {
                          c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_whole_norm_kv_write": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
                                c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "ri_talking_attention": [c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
-                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
-                             c_void_p, c_void_p],
+    "ri_talking_attention_shares": [c_int, c_int],
+    "ri_talking_attention": [c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p,
+                             c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                             c_float, c_void_p, c_void_p, c_void_p, c_void_p],
     "ri_shift_mix": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_shift_keep": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_timemix_max_dim": [],
     "ri_tanh_rows": [c_void_p, c_int, c_void_p, ctypes.c_long, c_void_p],
     "ri_timemix_scan": [c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                         c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ri_timemix_scan_cols_fits": [c_int],
+    "ri_timemix_scan_cols": [c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                             c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                             c_void_p],
     "ri_causal_conv_silu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                             c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_ssd_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_ssd_scan_cols_fits": [c_int, c_int],
+    "ri_ssd_scan_cols": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_group_rms_norm": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_void_p],
 }
 
@@ -1359,20 +1367,29 @@ def whole_norm_kv_write(proj, q_off: int, k_off: int, q_gain, k_gain, eps: float
           code(k_pages.dtype), k_pages.shape[2], tokens, heads, kv_heads, dim, _stream())
 
 
-def talking_attention(out, out_off: int, out_scale: float, proj, q_off: int, k_pages, v_pages, tok_pos, tok_seq, page_table,
-                      heads: int, kv_heads: int, dim: int, window: int | None, scale: float, r1, r2, talk) -> None:
+def talking_attention_shares(tokens: int, longest: int) -> int:
+    """Into how many shares a step of ``tokens`` tokens that see up to ``longest`` keys each cuts its walk over the keys."""
+    return _get("ri_talking_attention_shares")(int(tokens), int(longest))
+
+
+def talking_attention(proj, q_off: int, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, kv_heads: int, dim: int,
+                      window: int | None, scale: float, r1, r2, talk, shares: int = 1) -> torch.Tensor:
     """Windowed attention of every new token over its sequence's pages with the distance bias ``r1_h ln(1 + r2_h (i - j))``
-    taken off the scores and the heads' weights mixed by ``talk [heads, heads]`` after the softmax; the heads' results,
-    times ``out_scale``, go to the columns ``out_off ..`` of ``out``.  ``r1``/``r2`` and ``talk`` may be None."""
+    taken off the scores and the heads' weights mixed by ``talk [heads, heads]`` after the softmax: ``[T, heads * dim]``, the
+    heads side by side.  ``r1``/``r2`` and ``talk`` may be None.  With ``shares > 1`` (a step of few tokens) the walk over the
+    keys is cut into that many shares that run side by side, and the result is float32."""
     tokens = proj.shape[0]
-    if out.shape[0] != tokens or out.dtype != proj.dtype:
-        raise ShapeError(f"talking_attention: out {list(out.shape)} {out.dtype} for rows {list(proj.shape)} {proj.dtype}")
-    _call("ri_talking_attention", _dev(out, "out"), out.shape[1], int(out_off), float(out_scale), _dev(proj, "proj"),
-          code(proj.dtype), proj.shape[1], int(q_off), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), code(k_pages.dtype),
-          _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+    width = heads * dim
+    stats = torch.empty((tokens, heads, 2), dtype=torch.float32, device=proj.device)
+    out = (torch.empty((tokens, width), dtype=proj.dtype, device=proj.device) if shares == 1
+           else torch.empty((shares, tokens, width), dtype=torch.float32, device=proj.device))
+    _call("ri_talking_attention", _dev(out, "out"), code(out.dtype), width, 0, 1.0, int(shares), _dev(stats, "stats"),
+          _dev(proj, "proj"), code(proj.dtype), proj.shape[1], int(q_off), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
+          code(k_pages.dtype), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], tokens, heads, kv_heads, dim, k_pages.shape[2],
           int(window or 0), float(scale), _opt(r1, "r1", torch.float32, (heads,)), _opt(r2, "r2", torch.float32, (heads,)),
           _opt(talk, "talk", torch.float32, (heads, heads)), _stream())
+    return out if shares == 1 else sum_parts(out, torch.float32)
 
 
 # ---------------------------------------------------------------- time mixing
@@ -1408,10 +1425,12 @@ def shift_keep(kept, x32, cu_seqlens, slots) -> None:
 
 
 def timemix_scan(out, out_off: int, out_scale: float, r, k, v, g, z, w0, u, gain, eps: float, state, cu_seqlens, slots,
-                 heads: int, dim: int) -> None:
+                 heads: int, dim: int, columns: bool | None = None) -> None:
     """The walk of the time mixing over every sequence's new tokens on ``state [slots, heads, dim, dim]`` (float32, in
     place); ``r, k, v, g [T, heads * dim]``, ``z`` float32 the decay's pre-activation without its bias ``w0``; the normed and
-    gated heads, times ``out_scale``, go to the columns ``out_off ..`` of ``out``."""
+    gated heads, times ``out_scale``, go to the columns ``out_off ..`` of ``out``.  ``columns``: the form in which a thread holds a
+    whole column of the state (heads of up to 128; the default where it fits), else the form that cuts the rows into slices;
+    the two differ by rounding alone."""
     tokens, width = r.shape
     seqs = slots.shape[0]
     for name, t in (("k", k), ("v", v), ("g", g)):
@@ -1419,6 +1438,16 @@ def timemix_scan(out, out_off: int, out_scale: float, r, k, v, g, z, w0, u, gain
             raise ShapeError(f"timemix_scan: {name} is {list(t.shape)} {t.dtype}, r {list(r.shape)} {r.dtype}")
     if width != heads * dim or tuple(state.shape[1:]) != (heads, dim, dim) or out.shape[0] != tokens or out.dtype != r.dtype:
         raise ShapeError(f"timemix_scan: rows of {width}, state {list(state.shape)}, out {list(out.shape)}")
+    fits = bool(_get("ri_timemix_scan_cols_fits")(dim))
+    if fits if columns is None else (columns and fits):
+        o = torch.empty((tokens, width), dtype=torch.float32, device=r.device)
+        _call("ri_timemix_scan_cols", _dev(out, "out"), out.shape[1], int(out_off), float(out_scale), _dev(o, "o"), _dev(r, "r"),
+              _dev(k, "k"), _dev(v, "v"), _dev(g, "g"), code(r.dtype), _dev(z, "z", torch.float32, (tokens, width)),
+              _dev(w0, "w0", torch.float32, (width,)), _dev(u, "u", torch.float32, (width,)),
+              _dev(gain, "gain", torch.float32, (width,)), float(eps), _dev(state, "state", torch.float32),
+              _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32), tokens, seqs, heads, dim,
+              _stream())
+        return
     _call("ri_timemix_scan", _dev(out, "out"), out.shape[1], int(out_off), float(out_scale), _dev(r, "r"), _dev(k, "k"),
           _dev(v, "v"), _dev(g, "g"), code(r.dtype), _dev(z, "z", torch.float32, (tokens, width)),
           _dev(w0, "w0", torch.float32, (width,)), _dev(u, "u", torch.float32, (width,)),
@@ -1449,16 +1478,20 @@ def causal_conv_silu(proj, col0: int, channels: int, taps_w, bias, tails, tok_se
 
 
 def ssd_scan(xbc, b_off: int, c_off: int, proj, z_off: int, dt_off: int, dt_bias, a_log, d_skip, state, cu_seqlens, slots,
-             heads: int, groups: int, n: int, vdim: int) -> torch.Tensor:
+             heads: int, groups: int, n: int, vdim: int, columns: bool | None = None) -> torch.Tensor:
     """float32 ``[T, heads * vdim]``: the walk ``S <- exp(-exp(A_log) dt) S + dt B x^T``, ``y = S^T C + D x`` over every
     sequence's new tokens on ``state [slots, heads, n, vdim]`` (float32, in place), times ``silu(z)``; x, B and C are
-    columns of ``xbc`` (float32), z and the raw step sizes columns of ``proj``."""
+    columns of ``xbc`` (float32), z and the raw step sizes columns of ``proj``.  ``columns``: the form in which a thread holds a
+    whole column of the state (states of up to 128 rows; the default where it fits), else the form that cuts the rows into
+    slices; the two differ by rounding alone."""
     tokens, channels = xbc.shape
     seqs = slots.shape[0]
     if tuple(state.shape[1:]) != (heads, n, vdim) or proj.shape[0] != tokens:
         raise ShapeError(f"ssd_scan: state {list(state.shape)} for {heads} heads of {n} x {vdim}")
     out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=xbc.device)
-    _call("ri_ssd_scan", _dev(out, "out"), _dev(xbc, "xbc", torch.float32), channels, int(b_off), int(c_off), _dev(proj, "proj"),
+    fits = bool(_get("ri_ssd_scan_cols_fits")(n, vdim))
+    columns = fits if columns is None else (columns and fits)
+    _call("ri_ssd_scan_cols" if columns else "ri_ssd_scan", _dev(out, "out"), _dev(xbc, "xbc", torch.float32), channels, int(b_off), int(c_off), _dev(proj, "proj"),
           code(proj.dtype), proj.shape[1], int(z_off), int(dt_off), _opt(dt_bias, "dt_bias", torch.float32, (heads,)),
           _dev(a_log, "a_log", torch.float32, (heads,)), _opt(d_skip, "d_skip", torch.float32, (heads,)),
           _dev(state, "state", torch.float32), _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)),

@@ -85,15 +85,12 @@ class TalkingAttention(Mixer):
             ops.whole_norm_kv_write(proj, 0, self.q_width, self.q_gain, self.k_gain, self.eps, ctx.tok_pos, ctx.tok_seq,
                                     page_table, store.k_pages, store.v_pages, self.heads, self.kv_heads, self.dim)
         with profiler.section(profiler.ATTENTION):
-            if self.gate:
-                o = torch.empty((proj.shape[0], self.out_width), dtype=proj.dtype, device=proj.device)
-                ops.talking_attention(o, 0, 1.0, proj, 0, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table,
-                                      self.heads, self.kv_heads, self.dim, self.window, self.scale, self.r1, self.r2, self.mix)
-                ops.gate_rows(out, out_col, o, proj, self.q_width + self.k_width, out_scale, ops.GATE_SIGMOID)
-            else:
-                ops.talking_attention(out, out_col, out_scale, proj, 0, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq,
-                                      page_table, self.heads, self.kv_heads, self.dim, self.window, self.scale, self.r1, self.r2,
-                                      self.mix)
+            # a step of few tokens cuts its walk over the keys into shares that run side by side
+            longest = min(ctx.max_len, self.window) if self.window else ctx.max_len
+            shares = 1 if rt.dtype == torch.float32 or rt.invariant else ops.talking_attention_shares(proj.shape[0], longest)
+            o = ops.talking_attention(proj, 0, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
+                                      self.kv_heads, self.dim, self.window, self.scale, self.r1, self.r2, self.mix, shares)
+            ops.gate_rows(out, out_col, o, proj if self.gate else None, self.q_width + self.k_width, out_scale, ops.GATE_SIGMOID)
 
     def forward(self, x, ctx, store, page_table):
         heads = torch.empty((x.shape[0], self.out_width), dtype=self.rt.dtype, device=self.rt.device)

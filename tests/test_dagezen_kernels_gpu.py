@@ -171,11 +171,11 @@ def test_latent_attention_through_every_cut(ops, heads, dim, rot, vdim, rank):
 
 
 # ---------------------------------------------------------------- the windowed attention whose heads talk
-@pytest.mark.parametrize("heads, kv_heads, dim, window", [(4, 2, 12, 9), (3, 3, 20, 33), (6, 1, 8, 70)])
-def test_talking_attention_through_every_cut(ops, heads, kv_heads, dim, window):
+@pytest.mark.parametrize("heads, kv_heads, dim, window, shares", [(4, 2, 12, 9, 1), (3, 3, 20, 33, 2), (6, 1, 8, 70, 1), (20, 2, 16, None, 3)])
+def test_talking_attention_through_every_cut(ops, heads, kv_heads, dim, window, shares):
     rng = np.random.default_rng(4)
     width, eps, scale = 36, 1e-5, 0.4
-    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale, "mask": {"size": window}}
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale, "mask": {"size": window or 10 ** 6}}
     w = {"q": rng.standard_normal((heads * dim, width)) / 3, "k": rng.standard_normal((kv_heads * dim, width)) / 3,
          "q.norm": 1 + 0.1 * rng.standard_normal(heads * dim), "k.norm": 1 + 0.1 * rng.standard_normal(kv_heads * dim),
          "r1": rng.random(heads), "r2": rng.random(heads) * 3, "talk": np.eye(heads) + 0.3 * rng.standard_normal((heads, heads)),
@@ -193,9 +193,8 @@ def test_talking_attention_through_every_cut(ops, heads, kv_heads, dim, window):
         qw, kw = heads * dim, kv_heads * dim
         ops.whole_norm_kv_write(proj, 0, qw, t(w["q.norm"]), t(w["k.norm"]), eps, st["tok_pos"], st["tok_seq"], st["table"],
                                 k_pages, v_pages, heads, kv_heads, dim)
-        o = guarded(torch.zeros((len(x), qw), device=DEV))
-        ops.talking_attention(o, 0, 1.0, proj, 0, k_pages, v_pages, st["tok_pos"], st["tok_seq"], st["table"], heads, kv_heads,
-                              dim, window, scale, t(w["r1"]), t(w["r2"]), t(w["talk"]))
+        o = ops.talking_attention(proj, 0, k_pages, v_pages, st["tok_pos"], st["tok_seq"], st["table"], heads, kv_heads, dim,
+                                  window, scale, t(w["r1"]), t(w["r2"]), t(w["talk"]), shares)
         got = guarded(torch.zeros((len(x), qw + 3), device=DEV))
         ops.gate_rows(got, 3, o, proj, qw + kw, 0.5, ops.GATE_SIGMOID)
         want, at = [], 0
@@ -217,15 +216,15 @@ def test_a_key_at_the_windows_edge_counts_and_the_next_one_does_not(ops):
         k_pages[loud // PAGE, 0, loud % PAGE, :] = 30.0
         v_pages[loud // PAGE, 0, 0, loud % PAGE] = 1.0
         q = t(np.ones((1, heads * dim)))
-        o = guarded(torch.zeros((1, heads * dim), device=DEV))
-        ops.talking_attention(o, 0, 1.0, q, 0, k_pages, v_pages, t([n - 1], torch.int32), t([0], torch.int32),
-                              t([[0, 1, 2, 3]], torch.int32), heads, 1, dim, window, 1.0, None, None, None)
+        o = ops.talking_attention(q, 0, k_pages, v_pages, t([n - 1], torch.int32), t([0], torch.int32),
+                                  t([[0, 1, 2, 3]], torch.int32), heads, 1, dim, window, 1.0, None, None, None, 1 if seen else 2)
         assert (f64(o)[0, 0] > 0.99) == seen
 
 
 # ---------------------------------------------------------------- time mixing
-@pytest.mark.parametrize("heads, dim", [(3, 12), (2, 40), (1, 70)])
-def test_time_mixing_through_every_cut(ops, heads, dim):
+@pytest.mark.parametrize("columns", [True, False])
+@pytest.mark.parametrize("heads, dim", [(3, 12), (2, 40), (1, 70), (1, 130)])
+def test_time_mixing_through_every_cut(ops, heads, dim, columns):
     rng = np.random.default_rng(5)
     width, eps, rank = 30, 1e-5, 5
     hw = heads * dim
@@ -252,7 +251,7 @@ def test_time_mixing_through_every_cut(ops, heads, dim):
         z = t(np.tanh(mx[4] @ w["w1"].T) @ w["w2"].T)
         out = guarded(torch.zeros((len(x), hw + 2), device=DEV))
         ops.timemix_scan(out, 2, 0.7, r, k, v, g, z, t(w["w0"]), t(w["u"].reshape(-1)), t(w["norm"]), eps, state, st["cu"],
-                         st["slots"], heads, dim)
+                         st["slots"], heads, dim, columns)
         want, at = [], 0
         for s in st["seqs"]:
             n = sum(1 for r_ in st["rows"] if r_[0] == s)
@@ -263,8 +262,10 @@ def test_time_mixing_through_every_cut(ops, heads, dim):
 
 
 # ---------------------------------------------------------------- the state-space mixer
-@pytest.mark.parametrize("heads, vdim, n, groups, taps, parts", [(4, 12, 10, 2, 3, 2), (2, 20, 40, 1, 1, 5), (3, 8, 70, 3, 5, 1)])
-def test_state_space_mixer_through_every_cut(ops, heads, vdim, n, groups, taps, parts):
+@pytest.mark.parametrize("columns", [True, False])
+@pytest.mark.parametrize("heads, vdim, n, groups, taps, parts", [(4, 12, 10, 2, 3, 2), (2, 20, 40, 1, 1, 5), (3, 8, 70, 3, 5, 1),
+                                                                 (1, 70, 130, 1, 2, 1)])
+def test_state_space_mixer_through_every_cut(ops, heads, vdim, n, groups, taps, parts, columns):
     rng = np.random.default_rng(6)
     width, eps = 30, 1e-5
     inner = heads * vdim
@@ -285,7 +286,7 @@ def test_state_space_mixer_through_every_cut(ops, heads, vdim, n, groups, taps, 
         proj = t(x @ w["in"].T)
         xbc = ops.causal_conv_silu(proj, inner, channels, t(w["conv"]), t(w["conv.b"]), tails, st["tok_seq"], st["cu"], st["slots"])
         y = ops.ssd_scan(xbc, inner, inner + groups * n, proj, 0, inner + channels, t(w["dt_bias"]), t(w["A_log"]), t(w["D"]),
-                         state, st["cu"], st["slots"], heads, groups, n, vdim)
+                         state, st["cu"], st["slots"], heads, groups, n, vdim, columns)
         got = ops.group_rms_norm(y, t(w["norm"]), eps, parts, torch.float32)
         want, at = [], 0
         for s in st["seqs"]:
