@@ -412,6 +412,13 @@ int ri_latent_prepare(void* proj, int act_dtype, int stride, int q_off, int kv_o
 int ri_head_products(void* out, int out_dtype, int out_stride, int out_off, int out_head, const void* x, int x_dtype,
                      int x_stride, int x_off, int x_head, const void* w, int w_dtype, const void* gates, int g_stride,
                      int g_off, float scale, int tokens, int heads, int k, int n, int extra, void* stream);
+// The attention over the cached latent on the matrix cores (latent_mfma.hip): bfloat16, pages of 32, (key_dim, rank) one of
+// (576, 512), (288, 256), (160, 128).
+int ri_latent_attention_mfma_fits(int key_dim, int rank, int page_size);
+int ri_latent_attention_mfma(void* out, const void* q, int q_stride, const void* k_pages, const void* v_pages,
+                             const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table, int table_width,
+                             int tokens, int heads, int key_dim, int rank, int page_size, float scale, const float* sinks,
+                             void* stream);
 
 // ---- windowed attention whose heads talk (talking_attention.hip)
 int ri_whole_norm_kv_write(void* proj, int act_dtype, int stride, int q_off, int k_off, const float* q_gain,
@@ -438,7 +445,7 @@ int ri_timemix_scan(void* out, int out_stride, int out_off, float out_scale, con
                     const void* g, int act_dtype, const float* z, const float* w0, const float* u, const float* gain,
                     float eps, float* state, const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int dim,
                     void* stream);
-// The same walk with a thread a column of the state (heads of up to 128); o: float32 workspace [tokens, heads * dim].
+// The same walk with a wavefront on 16 columns of the state (heads of up to 128); o: float32 workspace [tokens, heads * dim].
 int ri_timemix_scan_cols_fits(int dim);
 int ri_timemix_scan_cols(void* out, int out_stride, int out_off, float out_scale, float* o, const void* r, const void* k,
                          const void* v, const void* g, int act_dtype, const float* z, const float* w0, const float* u,
@@ -454,7 +461,7 @@ int ri_ssd_scan(float* out, const float* xbc, int channels, int b_off, int c_off
                 int z_off, int dt_off, const float* dt_bias, const float* a_log, const float* d_skip, float* state,
                 const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int groups, int n, int vdim,
                 void* stream);
-// The same walk with a thread a column of the state, for states of up to 128 rows.
+// The same walk with a wavefront on 16 columns of the state, for states of up to 128 rows.
 int ri_ssd_scan_cols_fits(int n, int vdim);
 int ri_ssd_scan_cols(float* out, const float* xbc, int channels, int b_off, int c_off, const void* proj, int act_dtype, int stride,
                      int z_off, int dt_off, const float* dt_bias, const float* a_log, const float* d_skip, float* state,

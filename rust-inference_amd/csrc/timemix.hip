@@ -190,38 +190,44 @@ extern "C" int ri_timemix_scan(void* out, int out_stride, int out_off, float out
     return 0;
 }
 
-// ------------------------------------------------------------------ the walk, a thread a column
-// Heads of up to 128: a thread holds a whole column of the state in registers, so a token's sum over the rows needs no
-// other thread, and a workgroup is one wavefront on 64 columns of one (sequence, head).  Tokens are staged in LDS in
-// blocks of TM_BLOCK (r, k, the decay, v), the next block's loads asked for before the block in work is computed.  The
-// heads' results are written as they are, float32; the norm over a head and the gate are heads_norm_gate's.
+// ------------------------------------------------------------------ the walk, a wavefront on 16 columns
+// Heads of up to 128: a wavefront owns 16 columns of one (sequence, head), its lanes four slices of the rows of a column
+// each, the rows in registers; a token's sum over the rows is the lane's own sum (four partial sums, so that no addition
+// waits for the one before) and two exchanges between the lanes of a column.  A workgroup is one wavefront.  Tokens are
+// staged in LDS in blocks of TM_BLOCK (r, k, the decay, v), the next block's loads asked for before the block in work is
+// computed.  The heads' results are written as they are, float32; the norm over a head and the gate are
+// heads_norm_gate's.
 #define TM_BLOCK 8
+#define TM_COLS 16
 
-template <typename TA, int ROWS>
+template <typename TA, int RPL>                               // RPL: rows a lane holds, a multiple of 4
 __global__ void __launch_bounds__(64)
 timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, const TA* __restrict__ k, const TA* __restrict__ v,
                          const float* __restrict__ z, const float* __restrict__ w0, const float* __restrict__ u,
                          float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
                          int heads, int dim) {
+    constexpr int ROWS = 4 * RPL;
     __shared__ __attribute__((aligned(16))) float rs[2][TM_BLOCK][ROWS];
     __shared__ __attribute__((aligned(16))) float ks[2][TM_BLOCK][ROWS];
     __shared__ __attribute__((aligned(16))) float ws[2][TM_BLOCK][ROWS];
-    __shared__ __attribute__((aligned(16))) float us[ROWS];
-    __shared__ float vs[2][TM_BLOCK][64];
+    __shared__ float vs[2][TM_BLOCK][TM_COLS];
     const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int c = blockIdx.z * 64 + lane;
+    const int col = lane & 15, slice = lane >> 4, row0 = slice * RPL;
+    const int c = blockIdx.z * TM_COLS + col;
     const bool has_col = c < dim;
     const int cc = has_col ? c : dim - 1;                     // a column pulled back inside the head: loads are issued anyway
     const int width = heads * dim;
     float* sp = state + (((size_t)slots[seq] * heads + h) * dim) * dim + cc;
-    float st[ROWS];
+    float st[RPL], ub[RPL];
 #pragma unroll
-    for (int i = 0; i < ROWS; ++i) st[i] = i < dim ? sp[(size_t)i * dim] : 0.f;
-    for (int i = lane; i < ROWS; i += 64) us[i] = i < dim ? u[h * dim + i] : 0.f;
+    for (int i = 0; i < RPL; ++i) {
+        st[i] = row0 + i < dim ? sp[(size_t)(row0 + i) * dim] : 0.f;
+        ub[i] = row0 + i < dim ? u[h * dim + row0 + i] : 0.f;
+    }
     const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
     constexpr int PER = (TM_BLOCK * ROWS + 63) / 64;          // elements of each of r, k and the decay that a lane stages
 
-    float pre_r[PER], pre_k[PER], pre_w[PER], pre_v[TM_BLOCK];
+    float pre_r[PER], pre_k[PER], pre_w[PER], pre_v0 = 0.f, pre_v1 = 0.f;
     auto fetch = [&](int tb) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
@@ -233,8 +239,9 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
             pre_k[i] = in ? to_f32(k[at]) : 0.f;
             pre_w[i] = in ? z[at] + w0[h * dim + row] : 0.f;
         }
-#pragma unroll
-        for (int tt = 0; tt < TM_BLOCK; ++tt) pre_v[tt] = to_f32(v[(size_t)min(tb + tt, t1 - 1) * width + (size_t)h * dim + cc]);
+        const int tt = (lane >> 4) & 3;
+        pre_v0 = to_f32(v[(size_t)min(tb + tt, t1 - 1) * width + (size_t)h * dim + cc]);
+        pre_v1 = to_f32(v[(size_t)min(tb + 4 + tt, t1 - 1) * width + (size_t)h * dim + cc]);
     };
     auto stage = [&](int buf) {
 #pragma unroll
@@ -247,8 +254,9 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
                 ws[buf][tt][row] = expf(-expf(pre_w[i]));
             }
         }
-#pragma unroll
-        for (int tt = 0; tt < TM_BLOCK; ++tt) vs[buf][tt][lane] = pre_v[tt];
+        const int tt = (lane >> 4) & 3;
+        vs[buf][tt][col] = pre_v0;
+        vs[buf][4 + tt][col] = pre_v1;
     };
     if (t0 < t1) {
         fetch(t0);
@@ -261,32 +269,34 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
         if (more) fetch(tb + TM_BLOCK);
         const int count = min(TM_BLOCK, t1 - tb);
         for (int tt = 0; tt < count; ++tt) {
-            const float vc = vs[buf][tt][lane];
-            float o = 0.f;
+            const float vc = vs[buf][tt][col];
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
-            for (int i = 0; i < ROWS; i += 4) {
-                const float4 r4 = *reinterpret_cast<const float4*>(&rs[buf][tt][i]);
-                const float4 k4 = *reinterpret_cast<const float4*>(&ks[buf][tt][i]);
-                const float4 w4 = *reinterpret_cast<const float4*>(&ws[buf][tt][i]);
-                const float4 u4 = *reinterpret_cast<const float4*>(&us[i]);
+            for (int i = 0; i < RPL; i += 4) {
+                const float4 r4 = *reinterpret_cast<const float4*>(&rs[buf][tt][row0 + i]);
+                const float4 k4 = *reinterpret_cast<const float4*>(&ks[buf][tt][row0 + i]);
+                const float4 w4 = *reinterpret_cast<const float4*>(&ws[buf][tt][row0 + i]);
                 float kv = k4.x * vc;
-                o += (st[i] + u4.x * kv) * r4.x;             st[i] = w4.x * st[i] + kv;
+                o0 += (st[i] + ub[i] * kv) * r4.x;               st[i] = w4.x * st[i] + kv;
                 kv = k4.y * vc;
-                o += (st[i + 1] + u4.y * kv) * r4.y;         st[i + 1] = w4.y * st[i + 1] + kv;
+                o1 += (st[i + 1] + ub[i + 1] * kv) * r4.y;       st[i + 1] = w4.y * st[i + 1] + kv;
                 kv = k4.z * vc;
-                o += (st[i + 2] + u4.z * kv) * r4.z;         st[i + 2] = w4.z * st[i + 2] + kv;
+                o2 += (st[i + 2] + ub[i + 2] * kv) * r4.z;       st[i + 2] = w4.z * st[i + 2] + kv;
                 kv = k4.w * vc;
-                o += (st[i + 3] + u4.w * kv) * r4.w;         st[i + 3] = w4.w * st[i + 3] + kv;
+                o3 += (st[i + 3] + ub[i + 3] * kv) * r4.w;       st[i + 3] = w4.w * st[i + 3] + kv;
             }
-            if (has_col) out[(size_t)(tb + tt) * width + (size_t)h * dim + c] = o;
+            float o = (o0 + o1) + (o2 + o3);
+            o += __shfl_xor(o, 16, RI_WAVE);                  // the four slices of a column
+            o += __shfl_xor(o, 32, RI_WAVE);
+            if (has_col && slice == 0) out[(size_t)(tb + tt) * width + (size_t)h * dim + c] = o;
         }
         if (more) stage(buf ^ 1);
         __syncthreads();
     }
     if (has_col) {
 #pragma unroll
-        for (int i = 0; i < ROWS; ++i)
-            if (i < dim) sp[(size_t)i * dim] = st[i];
+        for (int i = 0; i < RPL; ++i)
+            if (row0 + i < dim) sp[(size_t)(row0 + i) * dim] = st[i];
     }
 }
 
@@ -317,13 +327,13 @@ extern "C" int ri_timemix_scan_cols(void* out, int out_stride, int out_off, floa
                "timemix_scan_cols: %d tokens of %d sequences, %d heads of %d", tokens, seqs, heads, dim);
     RI_REQUIRE(out_off >= 0 && out_off + heads * dim <= out_stride, "timemix_scan_cols: column %d of rows of %d", out_off, out_stride);
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "timemix_scan_cols: dtype %d", act_dtype);
-    const dim3 grid(seqs, heads, (dim + 63) / 64);
+    const dim3 grid(seqs, heads, (dim + TM_COLS - 1) / TM_COLS);
     hipStream_t s = (hipStream_t)stream;
 #define RI_GO(TA, ROWS)                                                                                                 \
     timemix_scan_cols_kernel<TA, ROWS><<<grid, 64, 0, s>>>(o, (const TA*)r, (const TA*)k, (const TA*)v, z, w0, u, state, \
                                                            cu_seqlens, slots, heads, dim)
 #define RI_BY_ROWS(TA)                                                                                                  \
-    if (dim <= 16) RI_GO(TA, 16); else if (dim <= 32) RI_GO(TA, 32); else if (dim <= 64) RI_GO(TA, 64); else RI_GO(TA, 128)
+    if (dim <= 16) RI_GO(TA, 4); else if (dim <= 32) RI_GO(TA, 8); else if (dim <= 64) RI_GO(TA, 16); else RI_GO(TA, 32)
     if (act_dtype == RI_F32) {
         RI_BY_ROWS(float);
         heads_norm_gate_kernel<float><<<dim3(tokens, heads), 64, 0, s>>>((float*)out, out_stride, out_off, out_scale, o, gain,

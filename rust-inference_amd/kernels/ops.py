@@ -134,6 +134,9 @@ _SIGNATURES = {
     "ri_softcap_rows": [c_void_p, c_float, ctypes.c_long, c_void_p],
     "ri_latent_prepare": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_latent_attention_mfma_fits": [c_int, c_int, c_int],
+    "ri_latent_attention_mfma": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                 c_int, c_int, c_int, c_float, c_void_p, c_void_p],
     "ri_head_products": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
                          c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_whole_norm_kv_write": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
@@ -1330,6 +1333,27 @@ def latent_prepare(proj, q_off: int, kv_off: int, gain, eps: float, inv_freq, to
           _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
           code(k_pages.dtype), k_pages.shape[2], tokens, heads, dim, rot, rank, _stream())
+
+
+def latent_attention_mfma_fits(dtype, key_dim: int, rank: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and bool(_get("ri_latent_attention_mfma_fits")(key_dim, rank, page_size))
+
+
+def latent_attention_mfma(q, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, scale: float, sinks) -> torch.Tensor:
+    """bfloat16 ``[T, heads * rank]``: causal attention on the matrix cores of every new token's ``heads`` query rows (``q [T,
+    heads * key_dim]``) over its sequence's single key/value head (``k_pages [pages, 1, 32, key_dim]``, ``v_pages [pages, 1, rank,
+    32]``), with a sink per head in the softmax's denominator (or None)."""
+    tokens = q.shape[0]
+    key_dim, rank, page = k_pages.shape[3], v_pages.shape[2], k_pages.shape[2]
+    if k_pages.shape[1] != 1 or v_pages.shape[1] != 1 or v_pages.shape[3] != page or q.shape[1] != heads * key_dim:
+        raise ShapeError(f"latent_attention_mfma: q {list(q.shape)}, key pages {list(k_pages.shape)}, value pages {list(v_pages.shape)}")
+    out = torch.empty((tokens, heads * rank), dtype=torch.bfloat16, device=q.device)
+    _call("ri_latent_attention_mfma", _dev(out, "out"), _dev(q, "q", torch.bfloat16), q.shape[1],
+          _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
+          _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1], tokens, heads, key_dim, rank, page, float(scale),
+          _opt(sinks, "sinks", torch.float32, (heads,)), _stream())
+    return out
 
 
 def head_products(x, x_off: int, x_head: int, w, heads: int, k: int, n: int, extra: int = 0, out=None, out_off: int = 0,

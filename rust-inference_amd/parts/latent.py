@@ -97,8 +97,14 @@ class LatentAttention(Mixer):
             else:
                 raise ConfigError("a latent attention without unrotated elements has no kernel")
         with profiler.section(profiler.ATTENTION):
-            o = ops.attention(q, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads, 1,
-                              self.rank + self.rot, None, self.scale, sinks=self.sink)
+            if (not ctx.is_decode and not rt.invariant
+                    and ops.latent_attention_mfma_fits(q.dtype, self.rank + self.rot, self.rank, store.page_size)):
+                # prompts at the sizes the matrix cores take: a wavefront on 16 heads of a token walks the token's pages
+                o = ops.latent_attention_mfma(q, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
+                                              self.scale, self.sink)
+            else:
+                o = ops.attention(q, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads, 1,
+                                  self.rank + self.rot, None, self.scale, sinks=self.sink)
             heads = ops.head_products(o, 0, self.rank, self.w_uv, self.heads, self.rank, self.vdim,
                                       gates=proj if self.gate else None, g_off=kv_at + self.rank + self.rot)
         with profiler.section(profiler.OUT_PROJECTION):

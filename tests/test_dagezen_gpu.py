@@ -103,7 +103,7 @@ def settled(folder, tokens, dtype_name):
     """The number of positions before a router's first close call: two logits closer than the number format tells apart
     reliably.  From there on another implementation may rightly send a token elsewhere, and every state carries it on."""
     plain_logits(folder, tokens)
-    close = _settled[(folder, tuple(tokens))] < (1e-5 if dtype_name == "float32" else 2e-2)
+    close = _settled[(folder, tuple(tokens))] < (1e-5 if dtype_name == "float32" else 5e-2)
     return int(np.argmax(close)) if close.any() else len(tokens)
 
 

@@ -294,3 +294,22 @@ def test_state_space_mixer_through_every_cut(ops, heads, vdim, n, groups, taps, 
             want.append(P.mamba2_mixer(x[at:at + k], w, "", m, eps, states[s]))
             at += k
         close(got, np.concatenate(want), 3e-5, f"state-space mixer, step {counts}")
+
+
+# ---------------------------------------------------------------- the latent attention on the matrix cores
+@pytest.mark.parametrize("heads", [3, 20])
+def test_latent_attention_on_the_matrix_cores_is_the_general_kernel(ops, heads):
+    """bfloat16, key rows of 160 and value rows of 128: tokens at the start of a sequence, at a page's border and inside a
+    page, of two sequences whose pages lie in shuffled order, with sinks; against the general kernel on the same pages."""
+    rng = np.random.default_rng(11)
+    dk, rank, pages = 160, 128, 12
+    k_pages = guarded((torch.randn((pages, 1, PAGE, dk), device=DEV) * 0.5).to(torch.bfloat16))
+    v_pages = guarded(k_pages[:, :, :, :rank].transpose(2, 3).contiguous())
+    table = t([[5, 2, 9, 0], [7, 1, 3, 11]], torch.int32)
+    tok_seq, tok_pos = t([0, 0, 0, 1, 1, 1, 1], torch.int32), t([0, 31, 32, 5, 63, 64, 100], torch.int32)
+    q = guarded((torch.randn((7, heads * dk), device=DEV) * 0.5).to(torch.bfloat16))
+    sinks = t(rng.standard_normal(heads))
+    for sink in (sinks, None):
+        want = ops.attention(q, k_pages, v_pages, tok_pos, tok_seq, table, heads, 1, dk, None, 0.11, sinks=sink)
+        got = ops.latent_attention_mfma(q, k_pages, v_pages, tok_pos, tok_seq, table, heads, 0.11, sink)
+        close(got, f64(want), 1.2e-2, "matrix cores against the general kernel")
