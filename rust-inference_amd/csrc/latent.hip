@@ -89,42 +89,66 @@ extern "C" int ri_latent_prepare(void* proj, int act_dtype, int stride, int q_of
 
 // ------------------------------------------------------------------ a product per head
 #define HP_TOKENS 8          // tokens of a workgroup: a matrix element is loaded once for all of them
+#define HP_COLS 64           // result columns of a workgroup
+#define HP_SLICES 4          // slices of K that the four wavefronts of a workgroup take: a lane sums its slice's rows in order,
+                             // the slices meet through LDS in order
 
 template <typename TX, typename TW, typename TO>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(HP_COLS * HP_SLICES)
 head_products_kernel(TO* __restrict__ out, int out_stride, int out_off, int out_head, const TX* __restrict__ x, int x_stride,
                      int x_off, int x_head, const TW* __restrict__ w, const TX* __restrict__ gates, int g_stride, int g_off,
                      float scale, int tokens, int k, int n, int extra) {
-    extern __shared__ float xs[];                 // [HP_TOKENS][k + extra]
-    const int h = blockIdx.y, t0 = blockIdx.x * HP_TOKENS, tid = threadIdx.x;
+    extern __shared__ float lds[];
+    float* xs = lds;                                          // [HP_TOKENS][k + extra]
     const int width = k + extra;
-    for (int e = tid; e < HP_TOKENS * width; e += 256) {
-        const int tt = e / width, c = e % width, t = t0 + tt;
-        xs[e] = t < tokens ? to_f32(x[(size_t)t * x_stride + x_off + (size_t)h * x_head + c]) : 0.f;
+    float* red = xs + HP_TOKENS * width;                      // [HP_SLICES][HP_TOKENS][HP_COLS]
+    const int h = blockIdx.y, t0 = blockIdx.x * HP_TOKENS, tid = threadIdx.x;
+    const int lane = tid % HP_COLS, slice = tid / HP_COLS;
+    const int c = blockIdx.z * HP_COLS + lane;
+    for (int e = tid; e < HP_TOKENS * width; e += HP_COLS * HP_SLICES) {
+        const int tt = e / width, col = e % width, t = t0 + tt;
+        xs[e] = t < tokens ? to_f32(x[(size_t)t * x_stride + x_off + (size_t)h * x_head + col]) : 0.f;
     }
     __syncthreads();
-    const TW* wh = w + (size_t)h * k * n;
-    for (int c = tid; c < n + extra; c += 256) {
-        float acc[HP_TOKENS];
+    float acc[HP_TOKENS];
 #pragma unroll
-        for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = 0.f;
-        if (c < n) {
-            for (int r = 0; r < k; ++r) {
-                const float wv = to_f32(wh[(size_t)r * n + c]);
+    for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = 0.f;
+    if (c < n) {
+        const TW* wc = w + (size_t)h * k * n + c;
+        const int per = (k + HP_SLICES - 1) / HP_SLICES;      // rows of a slice
+        const int r0 = slice * per, r1 = min(k, r0 + per);
+        int r = r0;
+        for (; r + 8 <= r1; r += 8) {                         // eight loads asked for before the first is used
+            float wv[8];
 #pragma unroll
-                for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] += xs[tt * width + r] * wv;
-            }
-        } else {
+            for (int i = 0; i < 8; ++i) wv[i] = to_f32(wc[(size_t)(r + i) * n]);
 #pragma unroll
-            for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = xs[tt * width + k + (c - n)];
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] += xs[tt * width + r + i] * wv[i];
         }
+        for (; r < r1; ++r) {
+            const float wv = to_f32(wc[(size_t)r * n]);
+#pragma unroll
+            for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] += xs[tt * width + r] * wv;
+        }
+    } else if (c < n + extra && slice == 0) {
+#pragma unroll
+        for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = xs[tt * width + k + (c - n)];
+    }
+#pragma unroll
+    for (int tt = 0; tt < HP_TOKENS; ++tt) red[(slice * HP_TOKENS + tt) * HP_COLS + lane] = acc[tt];
+    __syncthreads();
+    if (slice == 0 && c < n + extra) {
 #pragma unroll
         for (int tt = 0; tt < HP_TOKENS; ++tt) {
             const int t = t0 + tt;
             if (t >= tokens) break;
+            float v = red[tt * HP_COLS + lane];
+            for (int sl = 1; sl < HP_SLICES; ++sl) v += red[(sl * HP_TOKENS + tt) * HP_COLS + lane];
             float g = scale;
             if (gates) g *= 1.f / (1.f + expf(-to_f32(gates[(size_t)t * g_stride + g_off + h])));
-            from_f32(out + (size_t)t * out_stride + out_off + (size_t)h * out_head + c, acc[tt] * g);
+            from_f32(out + (size_t)t * out_stride + out_off + (size_t)h * out_head + c, v * g);
         }
     }
 }
@@ -141,12 +165,13 @@ extern "C" int ri_head_products(void* out, int out_dtype, int out_stride, int ou
     RI_REQUIRE(!gates || (g_off >= 0 && g_off + heads <= g_stride), "head_products: gates at column %d of rows of %d", g_off, g_stride);
     RI_REQUIRE((x_dtype == RI_F32 || x_dtype == RI_BF16) && (w_dtype == RI_F32 || w_dtype == RI_BF16) &&
                (out_dtype == RI_F32 || out_dtype == RI_BF16), "head_products: dtypes %d, %d, %d", x_dtype, w_dtype, out_dtype);
-    const size_t lds = (size_t)HP_TOKENS * (k + extra) * sizeof(float);
-    RI_REQUIRE(lds <= 64 * 1024, "head_products: heads of %d exceed the kernel's 2048", k + extra);
+    const size_t lds = ((size_t)HP_TOKENS * (k + extra) + (size_t)HP_SLICES * HP_TOKENS * HP_COLS) * sizeof(float);
+    RI_REQUIRE(lds <= 64 * 1024, "head_products: heads of %d exceed the kernel's 1792", k + extra);
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid((tokens + HP_TOKENS - 1) / HP_TOKENS, heads);
+    const dim3 grid((tokens + HP_TOKENS - 1) / HP_TOKENS, heads, (n + extra + HP_COLS - 1) / HP_COLS);
+    RI_REQUIRE(grid.z <= 65535, "head_products: results of %d", n + extra);
 #define RI_GO(TX, TW, TO)                                                                                               \
-    head_products_kernel<TX, TW, TO><<<grid, 256, lds, s>>>((TO*)out, out_stride, out_off, out_head, (const TX*)x, x_stride, \
+    head_products_kernel<TX, TW, TO><<<grid, HP_COLS * HP_SLICES, lds, s>>>((TO*)out, out_stride, out_off, out_head, (const TX*)x, x_stride, \
                                                             x_off, x_head, (const TW*)w, (const TX*)gates, g_stride, g_off, \
                                                             scale, tokens, k, n, extra)
     if (x_dtype == RI_F32) {

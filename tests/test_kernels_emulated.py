@@ -61,6 +61,7 @@ SAMPLER_TESTS = os.path.join(HERE, "test_sampling_gpu.py")
 ZIDEPEL_TESTS = os.path.join(HERE, "test_zidepel_kernels_gpu.py")
 PISULORN_TESTS = os.path.join(HERE, "test_pisulorn_kernels_gpu.py")
 ZAKELORN_TESTS = os.path.join(HERE, "test_zakelorn_kernels_gpu.py")
+DAGEZEN_TESTS = os.path.join(HERE, "test_dagezen_kernels_gpu.py")
 PISULORN_SELECT = "not two_equal_keys and not many_sequences"      # not the 1,300 keys and the 512 workgroups on the emulated matrix cores (minutes)
 SAMPLER_SELECT = "(same_token_as_the_plain_sampler or top_p_drops) and not large"     # not the 151,936 entries, not the engine
 
@@ -83,6 +84,7 @@ def runs():
         "zidepel": _start([*PYTEST, *_workers(2), ZIDEPEL_TESTS]),
         "pisulorn": _start([*PYTEST, *_workers(2), PISULORN_TESTS, "-k", PISULORN_SELECT]),
         "zakelorn": _start([*PYTEST, *_workers(2), ZAKELORN_TESTS, "-k", "not thousands_of_keys"]),
+        "dagezen": _start([*PYTEST, *_workers(2), DAGEZEN_TESTS]),
         # (with one compute unit a prompt of 70 tokens already takes the form of the rotation kernel that gives a
         # wavefront four heads of a token)
         "zakelorn, one unit": _start([*PYTEST, ZAKELORN_TESTS, "-k", "rotation_unit_norm"], {"RI_EMU_COMPUTE_UNITS": "1"}),
@@ -136,6 +138,14 @@ def test_the_kernels_of_the_zakelorn_design_pass_on_the_cpu_build_between_guard_
     router and the experts' closing sum."""
     _passed(runs["zakelorn"])
     _passed(runs["zakelorn, one unit"], 12)
+
+
+def test_the_kernels_of_the_dagezen_design_pass_on_the_cpu_build_between_guard_pages(runs):
+    """tests/test_dagezen_kernels_gpu.py: the norm behind the residual sum, the clamped gate with biases, the experts
+    without gates, the cap, the latent attention's preparation, its products per head and its matrix-core form, the
+    windowed attention whose heads talk (whole and in shares of the keys), the time mixing and the state-space mixer in
+    both forms of their walks."""
+    _passed(runs["dagezen"])
 
 
 @pytest.mark.parametrize("units, tests", [("sixteen units", 7), ("one unit", 61)])
