@@ -433,6 +433,14 @@ int ri_talking_attention(void* out, int out_dtype, int out_stride, int out_off, 
                          int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
                          int table_width, int tokens, int heads, int kv_heads, int dim, int page_size, int window, float scale,
                          const float* r1, const float* r2, const float* talk, void* stream);
+// The same attention on the matrix cores (talking_mfma.hip): bfloat16, pages of 32, heads of 32, 64 or 128, a multiple of 8
+// heads up to 32; tiles: the sum over the sequences of their new tokens in sixteens, rounded up.
+int ri_talking_attention_mfma_fits(int heads, int kv_heads, int dim, int page_size);
+int ri_talking_attention_mfma(void* out, float* stats, const void* q, int q_stride, int q_off, const void* k_pages,
+                              const void* v_pages, const int32_t* tok_pos, const int32_t* cu_seqlens, int seqs,
+                              const int32_t* page_table, int table_width, int tiles, int heads, int kv_heads, int dim,
+                              int page_size, int window, float scale, const float* r1, const float* r2, const float* talk,
+                              void* stream);
 
 // ---- time mixing (timemix.hip)
 int ri_shift_mix(void* out, int out_dtype, const float* x, const float* kept, const float* mu, int n_mix,

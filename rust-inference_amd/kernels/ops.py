@@ -145,6 +145,10 @@ _SIGNATURES = {
     "ri_talking_attention": [c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                              c_float, c_void_p, c_void_p, c_void_p, c_void_p],
+    "ri_talking_attention_mfma_fits": [c_int, c_int, c_int, c_int],
+    "ri_talking_attention_mfma": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                  c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p,
+                                  c_void_p],
     "ri_shift_mix": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_shift_keep": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_timemix_max_dim": [],
@@ -1414,6 +1418,30 @@ def talking_attention(proj, q_off: int, k_pages, v_pages, tok_pos, tok_seq, page
           int(window or 0), float(scale), _opt(r1, "r1", torch.float32, (heads,)), _opt(r2, "r2", torch.float32, (heads,)),
           _opt(talk, "talk", torch.float32, (heads, heads)), _stream())
     return out if shares == 1 else sum_parts(out, torch.float32)
+
+
+def talking_attention_mfma_fits(dtype, heads: int, kv_heads: int, dim: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and bool(_get("ri_talking_attention_mfma_fits")(heads, kv_heads, dim, page_size))
+
+
+def talking_attention_mfma(proj, q_off: int, k_pages, v_pages, tok_pos, cu_seqlens, new_counts, page_table, heads: int,
+                           kv_heads: int, dim: int, window: int | None, scale: float, r1, r2, talk) -> torch.Tensor:
+    """The same attention on the matrix cores, for prompts in bfloat16: ``[T, heads * dim]``.  ``new_counts``: every
+    sequence's number of new tokens (the host's list), by which the launch counts its tiles of 16 tokens."""
+    tokens = proj.shape[0]
+    seqs = len(new_counts)
+    tiles = sum(-(-int(n) // 16) for n in new_counts)
+    out = torch.empty((tokens, heads * dim), dtype=torch.bfloat16, device=proj.device)
+    if tiles == 0:
+        return out
+    stats = torch.empty((tokens, heads, 2), dtype=torch.float32, device=proj.device)
+    _call("ri_talking_attention_mfma", _dev(out, "out"), _dev(stats, "stats"), _dev(proj, "proj", torch.bfloat16), proj.shape[1],
+          int(q_off), _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
+          _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), seqs,
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1], tiles, heads, kv_heads, dim, k_pages.shape[2],
+          int(window or 0), float(scale), _opt(r1, "r1", torch.float32, (heads,)), _opt(r2, "r2", torch.float32, (heads,)),
+          _opt(talk, "talk", torch.float32, (heads, heads)), _stream())
+    return out
 
 
 # ---------------------------------------------------------------- time mixing

@@ -88,8 +88,15 @@ class TalkingAttention(Mixer):
             # a step of few tokens cuts its walk over the keys into shares that run side by side
             longest = min(ctx.max_len, self.window) if self.window else ctx.max_len
             shares = 1 if rt.dtype == torch.float32 or rt.invariant else ops.talking_attention_shares(proj.shape[0], longest)
-            o = ops.talking_attention(proj, 0, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
-                                      self.kv_heads, self.dim, self.window, self.scale, self.r1, self.r2, self.mix, shares)
+            if (not ctx.is_decode and not rt.invariant and proj.shape[1] % 8 == 0
+                    and ops.talking_attention_mfma_fits(proj.dtype, self.heads, self.kv_heads, self.dim, store.page_size)):
+                # prompts at the sizes the matrix cores take: tiles of 16 tokens, both walks on them
+                o = ops.talking_attention_mfma(proj, 0, store.k_pages, store.v_pages, ctx.tok_pos, ctx.cu_seqlens, ctx.new_counts,
+                                               page_table, self.heads, self.kv_heads, self.dim, self.window, self.scale, self.r1,
+                                               self.r2, self.mix)
+            else:
+                o = ops.talking_attention(proj, 0, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
+                                          self.kv_heads, self.dim, self.window, self.scale, self.r1, self.r2, self.mix, shares)
             ops.gate_rows(out, out_col, o, proj if self.gate else None, self.q_width + self.k_width, out_scale, ops.GATE_SIGMOID)
 
     def forward(self, x, ctx, store, page_table):

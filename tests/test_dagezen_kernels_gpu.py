@@ -313,3 +313,27 @@ def test_latent_attention_on_the_matrix_cores_is_the_general_kernel(ops, heads):
         want = ops.attention(q, k_pages, v_pages, tok_pos, tok_seq, table, heads, 1, dk, None, 0.11, sinks=sink)
         got = ops.latent_attention_mfma(q, k_pages, v_pages, tok_pos, tok_seq, table, heads, 0.11, sink)
         close(got, f64(want), 1.2e-2, "matrix cores against the general kernel")
+
+
+@pytest.mark.parametrize("heads, kv_heads, dim, window", [(8, 2, 32, 40), (16, 16, 32, None), (8, 1, 64, 33)])
+def test_talking_attention_on_the_matrix_cores_is_the_general_kernel(ops, heads, kv_heads, dim, window):
+    """bfloat16: two sequences whose pages lie in shuffled order, one that goes on from 37 cached tokens with 21 new ones
+    (two tiles, the second partial) and one that starts with 50; with the distance bias and the mixing matrix, and without;
+    against the general kernels on the same pages."""
+    rng = np.random.default_rng(12)
+    pages = 10
+    k_pages = guarded((torch.randn((pages, kv_heads, PAGE, dim), device=DEV) * 0.6).to(torch.bfloat16))
+    v_pages = guarded((torch.randn((pages, kv_heads, dim, PAGE), device=DEV) * 0.6).to(torch.bfloat16))
+    table = t([[5, 2, 9], [7, 1, 3]], torch.int32)
+    counts, starts = [21, 50], [37, 0]
+    tok_seq = t([0] * 21 + [1] * 50, torch.int32)
+    tok_pos = t(list(range(37, 58)) + list(range(50)), torch.int32)
+    cu = t([0, 21, 71], torch.int32)
+    proj = guarded((torch.randn((71, heads * dim + 16), device=DEV) * 0.6).to(torch.bfloat16))
+    r1, r2 = t(rng.random(heads)), t(rng.random(heads) * 3)
+    talk = t(np.eye(heads) + 0.3 * rng.standard_normal((heads, heads)))
+    for a, b, c in ((r1, r2, talk), (None, None, None)):
+        want = ops.talking_attention(proj, 8, k_pages, v_pages, tok_pos, tok_seq, table, heads, kv_heads, dim, window, 0.2, a, b, c)
+        got = ops.talking_attention_mfma(proj, 8, k_pages, v_pages, tok_pos, cu, counts, table, heads, kv_heads, dim, window, 0.2,
+                                         a, b, c)
+        close(got, f64(want), 1.5e-2, "matrix cores against the general kernels")
