@@ -50,6 +50,84 @@ scaled_sum_norm_kernel(float* __restrict__ residual, TA* __restrict__ act, const
     }
 }
 
+// 16 bytes of float32 or 8 of bfloat16 at once, as four floats.
+__device__ __forceinline__ float4 pn_ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 pn_ld4(const bf16_t* p) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xFFFF0000u), __uint_as_float(w.y << 16),
+                       __uint_as_float(w.y & 0xFFFF0000u));
+}
+__device__ __forceinline__ void pn_st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void pn_st4(bf16_t* p, float4 v) {
+    uint2 w;
+    w.x = pack_bf16x2(v.x, v.y);
+    w.y = pack_bf16x2(v.z, v.w);
+    *reinterpret_cast<uint2*>(p) = w;
+}
+
+// The same for rows of up to 1,024 * VPT elements, a multiple of 4: a thread asks for all its 16-byte pieces of the
+// residual and of every part of y up front and keeps them in registers, so that a row is one trip to memory; the parts
+// are added in their order, the row's sums taken in an order that the width alone fixes.
+template <typename TY, typename TA, int VPT>
+__global__ void __launch_bounds__(256)
+scaled_sum_norm_vec_kernel(float* __restrict__ residual, TA* __restrict__ act, const TY* __restrict__ y, int parts,
+                           size_t part_stride, const float* __restrict__ y_bias, float alpha, const float* __restrict__ gain,
+                           const float* __restrict__ bias, float eps, int kind, int dim) {
+    __shared__ float scratch[16];
+    const size_t at = (size_t)blockIdx.x * dim;
+    float4 v[VPT];
+    int col[VPT];
+    bool ok[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = (threadIdx.x + i * 256) * 4;
+        ok[i] = c < dim;
+        col[i] = ok[i] ? c : 0;                              // a column pulled back inside the row: the load is issued anyway
+        const float4 r = pn_ld4(residual + at + col[i]);
+        const float4 w = pn_ld4(y + at + col[i]);
+        v[i] = make_float4(w.x, w.y, w.z, w.w);
+        for (int p = 1; p < parts; ++p) {
+            const float4 u = pn_ld4(y + p * part_stride + at + col[i]);
+            v[i] = make_float4(v[i].x + u.x, v[i].y + u.y, v[i].z + u.z, v[i].w + u.w);
+        }
+        if (y_bias) {
+            const float4 b = pn_ld4(y_bias + col[i]);
+            v[i] = make_float4(v[i].x + b.x, v[i].y + b.y, v[i].z + b.z, v[i].w + b.w);
+        }
+        v[i] = make_float4(v[i].x + alpha * r.x, v[i].y + alpha * r.y, v[i].z + alpha * r.z, v[i].w + alpha * r.w);
+    }
+    float mean = 0.f;
+    if (kind == PN_NORM_LAYER) {
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPT; ++i)
+            if (ok[i]) sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+        mean = block_sum(sum, scratch) / (float)dim;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        if (ok[i]) {
+            const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
+            ss += (a * a + b * b) + (c * c + d * d);
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)dim + eps);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        if (!ok[i]) continue;
+        const float4 g = pn_ld4(gain + col[i]);
+        float4 o = make_float4((v[i].x - mean) * inv * g.x, (v[i].y - mean) * inv * g.y, (v[i].z - mean) * inv * g.z,
+                               (v[i].w - mean) * inv * g.w);
+        if (bias) {
+            const float4 b = pn_ld4(bias + col[i]);
+            o = make_float4(o.x + b.x, o.y + b.y, o.z + b.z, o.w + b.w);
+        }
+        pn_st4(residual + at + col[i], o);
+        if (act) pn_st4(act + at + col[i], o);
+    }
+}
+
 extern "C" int ri_scaled_sum_norm(float* residual, void* act, int act_dtype, const void* y, int y_dtype, int parts,
                                   const float* y_bias, float alpha, const float* gain, const float* bias, float eps,
                                   int kind, int rows, int dim, void* stream) {
@@ -62,12 +140,21 @@ extern "C" int ri_scaled_sum_norm(float* residual, void* act, int act_dtype, con
     RI_REQUIRE(parts == 1 || y_dtype == RI_F32, "scaled_sum_norm: parts of a product are float32");
     hipStream_t s = (hipStream_t)stream;
     const size_t lds = (size_t)dim * sizeof(float), stride = (size_t)rows * dim;
+#define RI_VEC(TY, TA, VPT)                                                                                             \
+    scaled_sum_norm_vec_kernel<TY, TA, VPT><<<rows, 256, 0, s>>>(residual, (TA*)act, (const TY*)y, parts, stride, y_bias, \
+                                                                 alpha, gain, bias, eps, kind, dim)
 #define RI_GO(TY, TA)                                                                                                   \
+    if (dim % 4 == 0 && dim <= 1024) RI_VEC(TY, TA, 1);                                                                 \
+    else if (dim % 4 == 0 && dim <= 2048) RI_VEC(TY, TA, 2);                                                            \
+    else if (dim % 4 == 0 && dim <= 4096) RI_VEC(TY, TA, 4);                                                            \
+    else if (dim % 4 == 0 && dim <= 8192) RI_VEC(TY, TA, 8);                                                            \
+    else                                                                                                                \
     scaled_sum_norm_kernel<TY, TA><<<rows, 256, lds, s>>>(residual, (TA*)act, (const TY*)y, parts, stride, y_bias, alpha, \
                                                           gain, bias, eps, kind, dim)
     if (y_dtype == RI_F32) { if (act_dtype == RI_F32) RI_GO(float, float); else RI_GO(float, bf16_t); }
     else                   { if (act_dtype == RI_F32) RI_GO(bf16_t, float); else RI_GO(bf16_t, bf16_t); }
 #undef RI_GO
+#undef RI_VEC
     RI_LAUNCH_CHECK("scaled_sum_norm");
     return 0;
 }

@@ -206,16 +206,31 @@ talking_mix_kernel(TO* __restrict__ out, int out_stride, int out_off, float out_
             if (valid) {
                 const TC* kr = k_pages + (((long)table[j / page_size] * kv_heads + kvh) * page_size + j % page_size) * (long)dim;
                 if (VEC) {
-                    for (int d = 0; d < dim; d += TkVec<TC>::N) {
-                        float kv[TkVec<TC>::N];
-                        TkVec<TC>::load(kr + d, kv);
+                    // (the heads behind n are the group's last head again: no branch inside the walk over the key, whose
+                    // loads go out two at a time)
+                    constexpr int N = TkVec<TC>::N;
+                    int d = 0;
+                    for (; d + 2 * N <= dim; d += 2 * N) {
+                        float ka[N], kb[N];
+                        TkVec<TC>::load(kr + d, ka);
+                        TkVec<TC>::load(kr + d + N, kb);
 #pragma unroll
                         for (int i = 0; i < TK_SUB; ++i) {
-                            if (i < n) {
-                                const float* qh = qs + (size_t)(g0 + i) * dim + d;
+                            const float* qh = qs + (size_t)(g0 + min(i, n - 1)) * dim + d;
 #pragma unroll
-                                for (int e = 0; e < TkVec<TC>::N; ++e) dots[i] += qh[e] * kv[e];
-                            }
+                            for (int e = 0; e < N; ++e) dots[i] += qh[e] * ka[e];
+#pragma unroll
+                            for (int e = 0; e < N; ++e) dots[i] += qh[N + e] * kb[e];
+                        }
+                    }
+                    for (; d < dim; d += N) {
+                        float ka[N];
+                        TkVec<TC>::load(kr + d, ka);
+#pragma unroll
+                        for (int i = 0; i < TK_SUB; ++i) {
+                            const float* qh = qs + (size_t)(g0 + min(i, n - 1)) * dim + d;
+#pragma unroll
+                            for (int e = 0; e < N; ++e) dots[i] += qh[e] * ka[e];
                         }
                     }
                 } else {
@@ -257,33 +272,51 @@ talking_mix_kernel(TO* __restrict__ out, int out_stride, int out_off, float out_
         __syncthreads();
         // the values: eight neighbouring keys of a channel lie side by side in a page
         const int jj_lo = max(lo, base) - base, jj_hi = min(qpos, base + TK_TILE - 1) - base;
+        if (page_size % 8 == 0) {
+            // eight keys at a time: their page looked up once, then the loads of all of a thread's results asked for
+            // before the first is used (a result behind the last is the last again, and dropped)
+            for (int j0 = jj_lo & ~7; j0 <= jj_hi; j0 += 8) {
+                const int jk = base + j0;
+                const long page_at = (long)table[jk / page_size] * kv_heads;
+                const int slot = jk % page_size;
 #pragma unroll
-        for (int i = 0; i < TK_ACCS; ++i) {
-            const int oc = tid + i * 256;
-            if (oc < results) {
-                const int h = oc / vdim, c = oc % vdim;
-                float a = acc[i];
-                if (page_size % 8 == 0) {
-                    for (int j0 = jj_lo & ~7; j0 <= jj_hi; j0 += 8) {
-                        const int jk = base + j0;
-                        const TC* vp = v_pages + (((long)table[jk / page_size] * kv_heads + h / share) * (long)vdim + c) * page_size +
-                                       jk % page_size;
-                        float vv[8];
-                        TkVec<TC>::load(vp, vv);
-                        if (TkVec<TC>::N == 4) TkVec<TC>::load(vp + 4, vv + 4);
-                        const float* mx = mixed + h * TK_TILE + j0;
+                for (int i0 = 0; i0 < TK_ACCS; i0 += 4) {
+                    if (tid + i0 * 256 >= results) break;          // (the same for the whole workgroup but its last threads)
+                    float vv[4][8];
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) a += mx[e] * vv[e];       // a key that is not seen has the weight 0
+                    for (int i = 0; i < 4; ++i) {
+                        const int oc = min(tid + (i0 + i) * 256, results - 1);
+                        const int h = oc / vdim, c = oc % vdim;
+                        const TC* vp = v_pages + ((page_at + h / share) * (long)vdim + c) * page_size + slot;
+                        TkVec<TC>::load(vp, vv[i]);
+                        if (TkVec<TC>::N == 4) TkVec<TC>::load(vp + 4, vv[i] + 4);
                     }
-                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int oc = min(tid + (i0 + i) * 256, results - 1);
+                        const float* mx = mixed + (oc / vdim) * TK_TILE + j0;
+                        float a = acc[i0 + i];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) a += mx[e] * vv[i][e];       // a key that is not seen has the weight 0
+                        acc[i0 + i] = a;
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TK_ACCS; ++i) {
+                const int oc = tid + i * 256;
+                if (oc < results) {
+                    const int h = oc / vdim, c = oc % vdim;
+                    float a = acc[i];
                     for (int jj = jj_lo; jj <= jj_hi; ++jj) {
                         const int jk = base + jj;
                         a += mixed[h * TK_TILE + jj] *
                              to_f32(v_pages[(((long)table[jk / page_size] * kv_heads + h / share) * (long)vdim + c) * page_size +
                                             jk % page_size]);
                     }
+                    acc[i] = a;
                 }
-                acc[i] = a;
             }
         }
         __syncthreads();                                   // before the next tile overwrites ps and mixed
