@@ -9,14 +9,14 @@
 //
 // The mixing needs every head's finished softmax, so the keys are walked twice: first each head's maximum and sum, a
 // workgroup per (token, head); then a workgroup per token makes, tile by tile, the weights of all heads, their mix and
-// the products with the values.  Tiles start at fixed multiples (256 keys in the first walk, 64 in the second), so the
+// the products with the values.  Tiles start at fixed multiples (256 keys in the first walk, 32 in the second), so the
 // order of every sum depends on the key's position alone.  A step of few tokens cuts the second walk's tiles into shares
 // that run side by side and whose float32 results the caller adds.  Scores, the logarithm, softmax statistics, the mix
 // and the accumulators are float32.
 #include "api.h"
 #include "common.h"
 
-#define TK_TILE 64
+#define TK_TILE 32
 #define TK_ACCS 16           // results a thread accumulates: heads * vdim <= 256 * TK_ACCS
 
 template <typename TA, typename TC>
@@ -153,7 +153,7 @@ talking_stats_kernel(float* __restrict__ stats, const TA* __restrict__ q, int q_
     }
 }
 
-// The second walk: a workgroup per token (and share of the key tiles) makes the weights of all heads for a tile of 64
+// The second walk: a workgroup per token (and share of the key tiles) makes the weights of all heads for a tile of 32
 // keys from the first walk's maxima and sums, mixes them, and adds the products with the values.  With more than one
 // share the results are partial sums (float32, [share][token][heads * dim]) that the caller adds.
 template <typename TA, typename TC, typename TO, bool VEC>
