@@ -186,29 +186,28 @@ extern "C" int ri_ssd_scan(float* out, const float* xbc, int channels, int b_off
 
 // ------------------------------------------------------------------ the walk, a wavefront on 16 columns
 // States of up to 128 rows: a wavefront owns 16 columns of one (sequence, head), its lanes four slices of the rows of a
-// column each, the rows in registers; a token's sum over the rows is the lane's own sum (four partial sums, so that no
+// column each (8 columns and eight slices for states above 64 rows), the rows in registers; a token's sum over the rows is the lane's own sum (four partial sums, so that no
 // addition waits for the one before) and two exchanges between the lanes of a column.  A workgroup is one wavefront.
 // Tokens are staged in LDS in blocks of SSD_BLOCK (B, C, x, the step size and decay, z), the next block's loads asked
 // for before the block in work is computed.  The order of a token's additions is fixed by the sizes alone.
 #define SSD_BLOCK 8
-#define SSD_COLS 16
 
-template <typename TA, int RPL>                               // RPL: rows a lane holds, a multiple of 4
+template <typename TA, int RPL, int SL>                       // RPL: rows a lane holds, a multiple of 4; SL: slices of rows, 4 or 8
 __global__ void __launch_bounds__(64)
 ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int channels, int b_off, int c_off,
                      const TA* __restrict__ proj, int stride, int z_off, int dt_off, const float* __restrict__ dt_bias,
                      const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ state,
                      const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots, int heads, int groups, int n,
                      int vdim) {
-    constexpr int ROWS = 4 * RPL;
+    constexpr int ROWS = SL * RPL, COLS = 64 / SL, TPP = 64 / COLS, PASSES = SSD_BLOCK / TPP;      // TPP: tokens whose x and z a pass fetches
     __shared__ __attribute__((aligned(16))) float bs[2][SSD_BLOCK][ROWS];
     __shared__ __attribute__((aligned(16))) float cs[2][SSD_BLOCK][ROWS];
-    __shared__ float xs[2][SSD_BLOCK][SSD_COLS];
-    __shared__ float zs[2][SSD_BLOCK][SSD_COLS];
+    __shared__ float xs[2][SSD_BLOCK][COLS];
+    __shared__ float zs[2][SSD_BLOCK][COLS];
     __shared__ float dts[2][SSD_BLOCK], decays[2][SSD_BLOCK];
     const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int col = lane & 15, slice = lane >> 4, row0 = slice * RPL;
-    const int c = blockIdx.z * SSD_COLS + col;
+    const int col = lane % COLS, slice = lane / COLS, row0 = slice * RPL;
+    const int c = blockIdx.z * COLS + col;
     const bool has_col = c < vdim;
     const int cc = has_col ? c : vdim - 1;                    // a column pulled back inside the head: loads are issued anyway
     const int group = h / (heads / groups), inner = heads * vdim;
@@ -220,7 +219,7 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
     const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
     constexpr int PER = (2 * SSD_BLOCK * ROWS + 63) / 64;     // B and C elements of a block a lane stages
 
-    float pre_bc[PER], pre_x0 = 0.f, pre_x1 = 0.f;
+    float pre_bc[PER], pre_x[PASSES], pre_z[PASSES], pre_raw = 0.f;
     auto fetch = [&](int tb) {                                // a block's loads, into registers
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
@@ -229,18 +228,12 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
             const int t = min(tb + tt, t1 - 1);
             pre_bc[i] = (r < n && which < 2) ? xbc[(size_t)t * channels + (which ? c_off : b_off) + group * n + r] : 0.f;
         }
-        {                                                     // x of 8 tokens x 16 columns, then z likewise: 128 a wavefront each
-            const int tt = (lane >> 4) & 3, cx = min((int)blockIdx.z * SSD_COLS + (lane & 15), vdim - 1);
-            const int ta = min(tb + tt, t1 - 1), tb2 = min(tb + 4 + tt, t1 - 1);
-            pre_x0 = xbc[(size_t)ta * channels + h * vdim + cx];
-            pre_x1 = xbc[(size_t)tb2 * channels + h * vdim + cx];
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {                 // x and z of the block's tokens for this wavefront's columns
+            const int t = min(tb + ps * TPP + slice, t1 - 1);
+            pre_x[ps] = xbc[(size_t)t * channels + h * vdim + cc];
+            pre_z[ps] = to_f32(proj[(size_t)t * stride + z_off + h * vdim + cc]);
         }
-    };
-    float pre_z0 = 0.f, pre_z1 = 0.f, pre_raw = 0.f;
-    auto fetch_z = [&](int tb) {
-        const int tt = (lane >> 4) & 3, cx = min((int)blockIdx.z * SSD_COLS + (lane & 15), vdim - 1);
-        pre_z0 = to_f32(proj[(size_t)min(tb + tt, t1 - 1) * stride + z_off + h * vdim + cx]);
-        pre_z1 = to_f32(proj[(size_t)min(tb + 4 + tt, t1 - 1) * stride + z_off + h * vdim + cx]);
         if (lane < SSD_BLOCK) pre_raw = to_f32(proj[(size_t)min(tb + lane, t1 - 1) * stride + dt_off + h]);
     };
     auto stage = [&](int buf) {                               // ... and from there into LDS
@@ -251,11 +244,11 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
             if (which == 0) bs[buf][tt][r] = pre_bc[i];
             else if (which == 1) cs[buf][tt][r] = pre_bc[i];
         }
-        const int tt = (lane >> 4) & 3;
-        xs[buf][tt][lane & 15] = pre_x0;
-        xs[buf][4 + tt][lane & 15] = pre_x1;
-        zs[buf][tt][lane & 15] = pre_z0;
-        zs[buf][4 + tt][lane & 15] = pre_z1;
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            xs[buf][ps * TPP + slice][col] = pre_x[ps];
+            zs[buf][ps * TPP + slice][col] = pre_z[ps];
+        }
         if (lane < SSD_BLOCK) {
             const float raw = pre_raw + bias;
             const float dt = raw > 20.f ? raw : log1pf(expf(raw));       // softplus: beyond 20 it is its argument to the last bit
@@ -265,7 +258,6 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
     };
     if (t0 < t1) {
         fetch(t0);
-        fetch_z(t0);
         stage(0);
     }
     __syncthreads();
@@ -274,7 +266,6 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
         const bool more = tb + SSD_BLOCK < t1;
         if (more) {
             fetch(tb + SSD_BLOCK);
-            fetch_z(tb + SSD_BLOCK);
         }
         const int count = min(SSD_BLOCK, t1 - tb);
         for (int tt = 0; tt < count; ++tt) {
@@ -291,7 +282,8 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
                 st[i + 3] = decay * st[i + 3] + b4.w * dx;     y3 += st[i + 3] * c4.w;
             }
             float y = (y0 + y1) + (y2 + y3);
-            y += __shfl_xor(y, 16, RI_WAVE);                  // the four slices of a column
+            if (SL == 8) y += __shfl_xor(y, 8, RI_WAVE);      // the slices of a column
+            y += __shfl_xor(y, 16, RI_WAVE);
             y += __shfl_xor(y, 32, RI_WAVE);
             y += skip * x;
             const float z = zs[buf][tt][col];
@@ -320,15 +312,16 @@ extern "C" int ri_ssd_scan_cols(float* out, const float* xbc, int channels, int 
     RI_REQUIRE(z_off >= 0 && dt_off >= 0 && z_off + heads * vdim <= stride && dt_off + heads <= stride,
                "ssd_scan_cols: columns %d and %d of rows of %d", z_off, dt_off, stride);
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "ssd_scan_cols: dtype %d", act_dtype);
-    const dim3 grid(seqs, heads, (vdim + SSD_COLS - 1) / SSD_COLS);
+    const int cols = n > 64 ? 8 : 16;
+    const dim3 grid(seqs, heads, (vdim + cols - 1) / cols);
     RI_REQUIRE(grid.z <= 65535, "ssd_scan_cols: heads of %d channels", vdim);
     hipStream_t s = (hipStream_t)stream;
-#define RI_GO(TA, RPL)                                                                                                  \
-    ssd_scan_cols_kernel<TA, RPL><<<grid, 64, 0, s>>>(out, xbc, channels, b_off, c_off, (const TA*)proj, stride, z_off,  \
+#define RI_GO(TA, RPL, SL)                                                                                              \
+    ssd_scan_cols_kernel<TA, RPL, SL><<<grid, 64, 0, s>>>(out, xbc, channels, b_off, c_off, (const TA*)proj, stride, z_off,  \
                                                       dt_off, dt_bias, a_log, d_skip, state, cu_seqlens, slots, heads,   \
                                                       groups, n, vdim)
 #define RI_BY_ROWS(TA)                                                                                                  \
-    if (n <= 16) RI_GO(TA, 4); else if (n <= 32) RI_GO(TA, 8); else if (n <= 64) RI_GO(TA, 16); else RI_GO(TA, 32)
+    if (n <= 16) RI_GO(TA, 4, 4); else if (n <= 32) RI_GO(TA, 8, 4); else if (n <= 64) RI_GO(TA, 16, 4); else RI_GO(TA, 16, 8)
     if (act_dtype == RI_F32) { RI_BY_ROWS(float); } else { RI_BY_ROWS(bf16_t); }
 #undef RI_BY_ROWS
 #undef RI_GO

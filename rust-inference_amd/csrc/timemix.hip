@@ -24,14 +24,13 @@ shift_mix_kernel(TA* __restrict__ out, const float* __restrict__ x, const float*
                  const float* __restrict__ mu, int n_mix, const int32_t* __restrict__ tok_seq,
                  const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots, int tokens, int width) {
     const int t = blockIdx.x;
+    const int d = blockIdx.y * 256 + threadIdx.x;             // a thread an element: a single token is many short workgroups
+    if (d >= width) return;
     const int seq = tok_seq[t];
     const float* before = t == cu_seqlens[seq] ? kept + (size_t)slots[seq] * width : x + (size_t)(t - 1) * width;
-    const float* here = x + (size_t)t * width;
-    for (int d = threadIdx.x; d < width; d += 256) {
-        const float h = here[d], delta = before[d] - h;
-        for (int s = 0; s < n_mix; ++s)
-            from_f32(out + ((size_t)s * tokens + t) * width + d, h + delta * mu[(size_t)s * width + d]);
-    }
+    const float h = x[(size_t)t * width + d], delta = before[d] - h;
+    for (int s = 0; s < n_mix; ++s)
+        from_f32(out + ((size_t)s * tokens + t) * width + d, h + delta * mu[(size_t)s * width + d]);
 }
 
 __global__ void __launch_bounds__(256)
@@ -46,13 +45,13 @@ shift_keep_kernel(float* __restrict__ kept, const float* __restrict__ x, const i
 extern "C" int ri_shift_mix(void* out, int out_dtype, const float* x, const float* kept, const float* mu, int n_mix,
                             const int32_t* tok_seq, const int32_t* cu_seqlens, const int32_t* slots, int tokens, int width,
                             void* stream) {
-    RI_REQUIRE(tokens > 0 && width > 0 && n_mix >= 1, "shift_mix: %d tokens of %d, %d mixes", tokens, width, n_mix);
+    RI_REQUIRE(tokens > 0 && width > 0 && width <= 65535 * 256 && n_mix >= 1, "shift_mix: %d tokens of %d, %d mixes", tokens, width, n_mix);
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "shift_mix: dtype %d", out_dtype);
     hipStream_t s = (hipStream_t)stream;
     if (out_dtype == RI_F32)
-        shift_mix_kernel<float><<<tokens, 256, 0, s>>>((float*)out, x, kept, mu, n_mix, tok_seq, cu_seqlens, slots, tokens, width);
+        shift_mix_kernel<float><<<dim3(tokens, (width + 255) / 256), 256, 0, s>>>((float*)out, x, kept, mu, n_mix, tok_seq, cu_seqlens, slots, tokens, width);
     else
-        shift_mix_kernel<bf16_t><<<tokens, 256, 0, s>>>((bf16_t*)out, x, kept, mu, n_mix, tok_seq, cu_seqlens, slots, tokens, width);
+        shift_mix_kernel<bf16_t><<<dim3(tokens, (width + 255) / 256), 256, 0, s>>>((bf16_t*)out, x, kept, mu, n_mix, tok_seq, cu_seqlens, slots, tokens, width);
     RI_LAUNCH_CHECK("shift_mix");
     return 0;
 }
@@ -192,28 +191,27 @@ extern "C" int ri_timemix_scan(void* out, int out_stride, int out_off, float out
 
 // ------------------------------------------------------------------ the walk, a wavefront on 16 columns
 // Heads of up to 128: a wavefront owns 16 columns of one (sequence, head), its lanes four slices of the rows of a column
-// each, the rows in registers; a token's sum over the rows is the lane's own sum (four partial sums, so that no addition
+// each (8 columns and eight slices for heads above 64: a token's walk over a lane's rows is what the wavefront waits for), the rows in registers; a token's sum over the rows is the lane's own sum (four partial sums, so that no addition
 // waits for the one before) and two exchanges between the lanes of a column.  A workgroup is one wavefront.  Tokens are
 // staged in LDS in blocks of TM_BLOCK (r, k, the decay, v), the next block's loads asked for before the block in work is
 // computed.  The heads' results are written as they are, float32; the norm over a head and the gate are
 // heads_norm_gate's.
 #define TM_BLOCK 8
-#define TM_COLS 16
 
-template <typename TA, int RPL>                               // RPL: rows a lane holds, a multiple of 4
+template <typename TA, int RPL, int SL>                       // RPL: rows a lane holds, a multiple of 4; SL: slices of rows, 4 or 8
 __global__ void __launch_bounds__(64)
 timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, const TA* __restrict__ k, const TA* __restrict__ v,
                          const float* __restrict__ z, const float* __restrict__ w0, const float* __restrict__ u,
                          float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
                          int heads, int dim) {
-    constexpr int ROWS = 4 * RPL;
+    constexpr int ROWS = SL * RPL, COLS = 64 / SL, TPP = 64 / COLS, PASSES = TM_BLOCK / TPP;      // TPP: tokens whose v a pass of the wavefront fetches
     __shared__ __attribute__((aligned(16))) float rs[2][TM_BLOCK][ROWS];
     __shared__ __attribute__((aligned(16))) float ks[2][TM_BLOCK][ROWS];
     __shared__ __attribute__((aligned(16))) float ws[2][TM_BLOCK][ROWS];
-    __shared__ float vs[2][TM_BLOCK][TM_COLS];
+    __shared__ float vs[2][TM_BLOCK][COLS];
     const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int col = lane & 15, slice = lane >> 4, row0 = slice * RPL;
-    const int c = blockIdx.z * TM_COLS + col;
+    const int col = lane % COLS, slice = lane / COLS, row0 = slice * RPL;
+    const int c = blockIdx.z * COLS + col;
     const bool has_col = c < dim;
     const int cc = has_col ? c : dim - 1;                     // a column pulled back inside the head: loads are issued anyway
     const int width = heads * dim;
@@ -227,7 +225,7 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
     const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
     constexpr int PER = (TM_BLOCK * ROWS + 63) / 64;          // elements of each of r, k and the decay that a lane stages
 
-    float pre_r[PER], pre_k[PER], pre_w[PER], pre_v0 = 0.f, pre_v1 = 0.f;
+    float pre_r[PER], pre_k[PER], pre_w[PER], pre_v[PASSES];
     auto fetch = [&](int tb) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
@@ -239,9 +237,9 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
             pre_k[i] = in ? to_f32(k[at]) : 0.f;
             pre_w[i] = in ? z[at] + w0[h * dim + row] : 0.f;
         }
-        const int tt = (lane >> 4) & 3;
-        pre_v0 = to_f32(v[(size_t)min(tb + tt, t1 - 1) * width + (size_t)h * dim + cc]);
-        pre_v1 = to_f32(v[(size_t)min(tb + 4 + tt, t1 - 1) * width + (size_t)h * dim + cc]);
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps)
+            pre_v[ps] = to_f32(v[(size_t)min(tb + ps * TPP + slice, t1 - 1) * width + (size_t)h * dim + cc]);
     };
     auto stage = [&](int buf) {
 #pragma unroll
@@ -254,9 +252,8 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
                 ws[buf][tt][row] = expf(-expf(pre_w[i]));
             }
         }
-        const int tt = (lane >> 4) & 3;
-        vs[buf][tt][col] = pre_v0;
-        vs[buf][4 + tt][col] = pre_v1;
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) vs[buf][ps * TPP + slice][col] = pre_v[ps];
     };
     if (t0 < t1) {
         fetch(t0);
@@ -286,7 +283,8 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
                 o3 += (st[i + 3] + ub[i + 3] * kv) * r4.w;       st[i + 3] = w4.w * st[i + 3] + kv;
             }
             float o = (o0 + o1) + (o2 + o3);
-            o += __shfl_xor(o, 16, RI_WAVE);                  // the four slices of a column
+            if (SL == 8) o += __shfl_xor(o, 8, RI_WAVE);      // the slices of a column
+            o += __shfl_xor(o, 16, RI_WAVE);
             o += __shfl_xor(o, 32, RI_WAVE);
             if (has_col && slice == 0) out[(size_t)(tb + tt) * width + (size_t)h * dim + c] = o;
         }
@@ -327,13 +325,14 @@ extern "C" int ri_timemix_scan_cols(void* out, int out_stride, int out_off, floa
                "timemix_scan_cols: %d tokens of %d sequences, %d heads of %d", tokens, seqs, heads, dim);
     RI_REQUIRE(out_off >= 0 && out_off + heads * dim <= out_stride, "timemix_scan_cols: column %d of rows of %d", out_off, out_stride);
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "timemix_scan_cols: dtype %d", act_dtype);
-    const dim3 grid(seqs, heads, (dim + TM_COLS - 1) / TM_COLS);
+    const int cols = dim > 64 ? 8 : 16;
+    const dim3 grid(seqs, heads, (dim + cols - 1) / cols);
     hipStream_t s = (hipStream_t)stream;
-#define RI_GO(TA, ROWS)                                                                                                 \
-    timemix_scan_cols_kernel<TA, ROWS><<<grid, 64, 0, s>>>(o, (const TA*)r, (const TA*)k, (const TA*)v, z, w0, u, state, \
+#define RI_GO(TA, ROWS, SL)                                                                                             \
+    timemix_scan_cols_kernel<TA, ROWS, SL><<<grid, 64, 0, s>>>(o, (const TA*)r, (const TA*)k, (const TA*)v, z, w0, u, state, \
                                                            cu_seqlens, slots, heads, dim)
 #define RI_BY_ROWS(TA)                                                                                                  \
-    if (dim <= 16) RI_GO(TA, 4); else if (dim <= 32) RI_GO(TA, 8); else if (dim <= 64) RI_GO(TA, 16); else RI_GO(TA, 32)
+    if (dim <= 16) RI_GO(TA, 4, 4); else if (dim <= 32) RI_GO(TA, 8, 4); else if (dim <= 64) RI_GO(TA, 16, 4); else RI_GO(TA, 16, 8)
     if (act_dtype == RI_F32) {
         RI_BY_ROWS(float);
         heads_norm_gate_kernel<float><<<dim3(tokens, heads), 64, 0, s>>>((float*)out, out_stride, out_off, out_scale, o, gain,
