@@ -268,26 +268,37 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
             fetch(tb + SSD_BLOCK);
         }
         const int count = min(SSD_BLOCK, t1 - tb);
-        for (int tt = 0; tt < count; ++tt) {
-            const float decay = decays[buf][tt], x = xs[buf][tt][col];
-            const float dx = dts[buf][tt] * x;
-            float y0 = 0.f, y1 = 0.f, y2 = 0.f, y3 = 0.f;
+        float part[SSD_BLOCK];                                // the lane's share of each token's sum: the exchanges wait for the block's end,
+#pragma unroll                                                // so that no token waits for the one before it
+        for (int tt = 0; tt < SSD_BLOCK; ++tt) {
+            part[tt] = 0.f;
+            if (tt < count) {
+                const float decay = decays[buf][tt];
+                const float dx = dts[buf][tt] * xs[buf][tt][col];
+                float y0 = 0.f, y1 = 0.f, y2 = 0.f, y3 = 0.f;
 #pragma unroll
-            for (int i = 0; i < RPL; i += 4) {
-                const float4 b4 = *reinterpret_cast<const float4*>(&bs[buf][tt][row0 + i]);
-                const float4 c4 = *reinterpret_cast<const float4*>(&cs[buf][tt][row0 + i]);
-                st[i] = decay * st[i] + b4.x * dx;             y0 += st[i] * c4.x;
-                st[i + 1] = decay * st[i + 1] + b4.y * dx;     y1 += st[i + 1] * c4.y;
-                st[i + 2] = decay * st[i + 2] + b4.z * dx;     y2 += st[i + 2] * c4.z;
-                st[i + 3] = decay * st[i + 3] + b4.w * dx;     y3 += st[i + 3] * c4.w;
+                for (int i = 0; i < RPL; i += 4) {
+                    const float4 b4 = *reinterpret_cast<const float4*>(&bs[buf][tt][row0 + i]);
+                    const float4 c4 = *reinterpret_cast<const float4*>(&cs[buf][tt][row0 + i]);
+                    st[i] = decay * st[i] + b4.x * dx;             y0 += st[i] * c4.x;
+                    st[i + 1] = decay * st[i + 1] + b4.y * dx;     y1 += st[i + 1] * c4.y;
+                    st[i + 2] = decay * st[i + 2] + b4.z * dx;     y2 += st[i + 2] * c4.z;
+                    st[i + 3] = decay * st[i + 3] + b4.w * dx;     y3 += st[i + 3] * c4.w;
+                }
+                part[tt] = (y0 + y1) + (y2 + y3);
             }
-            float y = (y0 + y1) + (y2 + y3);
+        }
+#pragma unroll
+        for (int tt = 0; tt < SSD_BLOCK; ++tt) {
+            float y = part[tt];
             if (SL == 8) y += __shfl_xor(y, 8, RI_WAVE);      // the slices of a column
             y += __shfl_xor(y, 16, RI_WAVE);
             y += __shfl_xor(y, 32, RI_WAVE);
-            y += skip * x;
-            const float z = zs[buf][tt][col];
-            if (has_col && slice == 0) out[(size_t)(tb + tt) * inner + h * vdim + c] = y * (z / (1.f + expf(-z)));
+            if (tt < count && has_col && slice == 0) {
+                y += skip * xs[buf][tt][col];
+                const float z = zs[buf][tt][col];
+                out[(size_t)(tb + tt) * inner + h * vdim + c] = y * (z / (1.f + expf(-z)));
+            }
         }
         if (more) stage(buf ^ 1);
         __syncthreads();

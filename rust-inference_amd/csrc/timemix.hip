@@ -265,28 +265,37 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
         const bool more = tb + TM_BLOCK < t1;
         if (more) fetch(tb + TM_BLOCK);
         const int count = min(TM_BLOCK, t1 - tb);
-        for (int tt = 0; tt < count; ++tt) {
-            const float vc = vs[buf][tt][col];
-            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+        float part[TM_BLOCK];                                 // the lane's share of each token's sum: the exchanges wait for the block's end,
+#pragma unroll                                                // so that no token waits for the one before it
+        for (int tt = 0; tt < TM_BLOCK; ++tt) {
+            part[tt] = 0.f;
+            if (tt < count) {
+                const float vc = vs[buf][tt][col];
+                float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
-            for (int i = 0; i < RPL; i += 4) {
-                const float4 r4 = *reinterpret_cast<const float4*>(&rs[buf][tt][row0 + i]);
-                const float4 k4 = *reinterpret_cast<const float4*>(&ks[buf][tt][row0 + i]);
-                const float4 w4 = *reinterpret_cast<const float4*>(&ws[buf][tt][row0 + i]);
-                float kv = k4.x * vc;
-                o0 += (st[i] + ub[i] * kv) * r4.x;               st[i] = w4.x * st[i] + kv;
-                kv = k4.y * vc;
-                o1 += (st[i + 1] + ub[i + 1] * kv) * r4.y;       st[i + 1] = w4.y * st[i + 1] + kv;
-                kv = k4.z * vc;
-                o2 += (st[i + 2] + ub[i + 2] * kv) * r4.z;       st[i + 2] = w4.z * st[i + 2] + kv;
-                kv = k4.w * vc;
-                o3 += (st[i + 3] + ub[i + 3] * kv) * r4.w;       st[i + 3] = w4.w * st[i + 3] + kv;
+                for (int i = 0; i < RPL; i += 4) {
+                    const float4 r4 = *reinterpret_cast<const float4*>(&rs[buf][tt][row0 + i]);
+                    const float4 k4 = *reinterpret_cast<const float4*>(&ks[buf][tt][row0 + i]);
+                    const float4 w4 = *reinterpret_cast<const float4*>(&ws[buf][tt][row0 + i]);
+                    float kv = k4.x * vc;
+                    o0 += (st[i] + ub[i] * kv) * r4.x;               st[i] = w4.x * st[i] + kv;
+                    kv = k4.y * vc;
+                    o1 += (st[i + 1] + ub[i + 1] * kv) * r4.y;       st[i + 1] = w4.y * st[i + 1] + kv;
+                    kv = k4.z * vc;
+                    o2 += (st[i + 2] + ub[i + 2] * kv) * r4.z;       st[i + 2] = w4.z * st[i + 2] + kv;
+                    kv = k4.w * vc;
+                    o3 += (st[i + 3] + ub[i + 3] * kv) * r4.w;       st[i + 3] = w4.w * st[i + 3] + kv;
+                }
+                part[tt] = (o0 + o1) + (o2 + o3);
             }
-            float o = (o0 + o1) + (o2 + o3);
+        }
+#pragma unroll
+        for (int tt = 0; tt < TM_BLOCK; ++tt) {
+            float o = part[tt];
             if (SL == 8) o += __shfl_xor(o, 8, RI_WAVE);      // the slices of a column
             o += __shfl_xor(o, 16, RI_WAVE);
             o += __shfl_xor(o, 32, RI_WAVE);
-            if (has_col && slice == 0) out[(size_t)(tb + tt) * width + (size_t)h * dim + c] = o;
+            if (tt < count && has_col && slice == 0) out[(size_t)(tb + tt) * width + (size_t)h * dim + c] = o;
         }
         if (more) stage(buf ^ 1);
         __syncthreads();
