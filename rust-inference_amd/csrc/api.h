@@ -453,10 +453,10 @@ int ri_timemix_scan(void* out, int out_stride, int out_off, float out_scale, con
                     const void* g, int act_dtype, const float* z, const float* w0, const float* u, const float* gain,
                     float eps, float* state, const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int dim,
                     void* stream);
-// The same walk with a wavefront on 16 columns of the state (heads of up to 128); o: float32 workspace [tokens, heads * dim].
+// The same walk with a wavefront on 16 columns of the state (heads of up to 128); o: float32 workspace [tokens, heads * dim]; z is overwritten with the decays.
 int ri_timemix_scan_cols_fits(int dim);
 int ri_timemix_scan_cols(void* out, int out_stride, int out_off, float out_scale, float* o, const void* r, const void* k,
-                         const void* v, const void* g, int act_dtype, const float* z, const float* w0, const float* u,
+                         const void* v, const void* g, int act_dtype, float* z, const float* w0, const float* u,
                          const float* gain, float eps, float* state, const int32_t* cu_seqlens, const int32_t* slots, int tokens,
                          int seqs, int heads, int dim, void* stream);
 

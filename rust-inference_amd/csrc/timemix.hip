@@ -201,7 +201,7 @@ extern "C" int ri_timemix_scan(void* out, int out_stride, int out_off, float out
 template <typename TA, int RPL, int SL>                       // RPL: rows a lane holds, a multiple of 4; SL: slices of rows, 4 or 8
 __global__ void __launch_bounds__(64)
 timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, const TA* __restrict__ k, const TA* __restrict__ v,
-                         const float* __restrict__ z, const float* __restrict__ w0, const float* __restrict__ u,
+                         const float* __restrict__ z, const float* __restrict__ u,
                          float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
                          int heads, int dim) {
     constexpr int ROWS = SL * RPL, COLS = 64 / SL, TPP = 64 / COLS, PASSES = TM_BLOCK / TPP;      // TPP: tokens whose v a pass of the wavefront fetches
@@ -235,7 +235,7 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
             const size_t at = (size_t)min(tb + tt, t1 - 1) * width + (size_t)h * dim + (in ? row : 0);
             pre_r[i] = in ? to_f32(r[at]) : 0.f;
             pre_k[i] = in ? to_f32(k[at]) : 0.f;
-            pre_w[i] = in ? z[at] + w0[h * dim + row] : 0.f;
+            pre_w[i] = in ? z[at] : 0.f;                     // the decay itself: timemix_decay has been over z
         }
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps)
@@ -249,7 +249,7 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
             if (tt < TM_BLOCK) {
                 rs[buf][tt][row] = pre_r[i];
                 ks[buf][tt][row] = pre_k[i];
-                ws[buf][tt][row] = expf(-expf(pre_w[i]));
+                ws[buf][tt][row] = pre_w[i];
             }
         }
 #pragma unroll
@@ -324,10 +324,17 @@ heads_norm_gate_kernel(TA* __restrict__ out, int out_stride, int out_off, float 
     }
 }
 
+// z <- exp(-exp(z + w0)) in place: every token's decays once, before the walk, whose sixteen wavefronts a head would each
+// take both exponentials again.
+__global__ void timemix_decay_kernel(float* __restrict__ z, const float* __restrict__ w0, long total, int width) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < total) z[e] = expf(-expf(z[e] + w0[e % width]));
+}
+
 extern "C" int ri_timemix_scan_cols_fits(int dim) { return dim >= 1 && dim <= 128; }
 
 extern "C" int ri_timemix_scan_cols(void* out, int out_stride, int out_off, float out_scale, float* o, const void* r,
-                                    const void* k, const void* v, const void* g, int act_dtype, const float* z, const float* w0,
+                                    const void* k, const void* v, const void* g, int act_dtype, float* z, const float* w0,
                                     const float* u, const float* gain, float eps, float* state, const int32_t* cu_seqlens,
                                     const int32_t* slots, int tokens, int seqs, int heads, int dim, void* stream) {
     RI_REQUIRE(tokens > 0 && seqs > 0 && heads > 0 && heads <= 65535 && ri_timemix_scan_cols_fits(dim),
@@ -337,8 +344,11 @@ extern "C" int ri_timemix_scan_cols(void* out, int out_stride, int out_off, floa
     const int cols = dim > 64 ? 8 : 16;
     const dim3 grid(seqs, heads, (dim + cols - 1) / cols);
     hipStream_t s = (hipStream_t)stream;
+    const long total = (long)tokens * heads * dim;
+    RI_REQUIRE((total + 255) / 256 <= 2147483647L, "timemix_scan_cols: %ld decays exceed one launch", total);
+    timemix_decay_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(z, w0, total, heads * dim);
 #define RI_GO(TA, ROWS, SL)                                                                                             \
-    timemix_scan_cols_kernel<TA, ROWS, SL><<<grid, 64, 0, s>>>(o, (const TA*)r, (const TA*)k, (const TA*)v, z, w0, u, state, \
+    timemix_scan_cols_kernel<TA, ROWS, SL><<<grid, 64, 0, s>>>(o, (const TA*)r, (const TA*)k, (const TA*)v, z, u, state,  \
                                                            cu_seqlens, slots, heads, dim)
 #define RI_BY_ROWS(TA)                                                                                                  \
     if (dim <= 16) RI_GO(TA, 4, 4); else if (dim <= 32) RI_GO(TA, 8, 4); else if (dim <= 64) RI_GO(TA, 16, 4); else RI_GO(TA, 16, 8)

@@ -1482,7 +1482,7 @@ def timemix_scan(out, out_off: int, out_scale: float, r, k, v, g, z, w0, u, gain
     place); ``r, k, v, g [T, heads * dim]``, ``z`` float32 the decay's pre-activation without its bias ``w0``; the normed and
     gated heads, times ``out_scale``, go to the columns ``out_off ..`` of ``out``.  ``columns``: the form in which a thread holds a
     whole column of the state (heads of up to 128; the default where it fits), else the form that cuts the rows into slices;
-    the two differ by rounding alone."""
+    the two differ by rounding alone.  The first form overwrites ``z`` with the decays."""
     tokens, width = r.shape
     seqs = slots.shape[0]
     for name, t in (("k", k), ("v", v), ("g", g)):

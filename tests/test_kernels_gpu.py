@@ -1005,10 +1005,10 @@ def test_kernels_refuse_what_they_cannot_do(ops):
             ops.swiglu(torch.zeros(2, 4))
     with pytest.raises(KernelError, match="1 to 8"):
         ops.gemv_bf16(torch.zeros(9, 16, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 16, dtype=torch.bfloat16, device=DEV))
-    with pytest.raises(KernelError, match="between 1 and 512"):
-        ops.attention(torch.zeros(1, 3 * 520, device=DEV), torch.zeros(1, 1, 32, 520, device=DEV),
-                      torch.zeros(1, 1, 520, 32, device=DEV), t([0], torch.int32), t([0], torch.int32),
-                      t([[0]], torch.int32), 1, 1, 520, None, 1.0)
+    with pytest.raises(KernelError, match="between 1 and 1024"):
+        ops.attention(torch.zeros(1, 3 * 1032, device=DEV), torch.zeros(1, 1, 32, 1032, device=DEV),
+                      torch.zeros(1, 1, 1032, 32, device=DEV), t([0], torch.int32), t([0], torch.int32),
+                      t([[0]], torch.int32), 1, 1, 1032, None, 1.0)
     with pytest.raises(ShapeError, match="contiguous"):
         ops.swiglu(torch.zeros(4, 8, device=DEV)[:, ::2])
 
