@@ -122,6 +122,12 @@ def test_clamped_gate_with_biases_and_the_experts_plain_activation_and_the_cap(o
     g = np.minimum(gu[:, :ff] + bg, limit)
     u = np.clip(gu[:, ff:] + bu, -limit, limit)
     close(ops.glu_clamped_bias(t(gu), t(bg), t(bu), limit), g * P.sigmoid(1.702 * g) * (u + 1), F32, "clamped gate")
+    wide = 2 * rng.standard_normal((3, 2 * 48))                       # bfloat16 rows of a multiple of 8: eight elements a thread
+    gb, ub = rng.standard_normal(48), rng.standard_normal(48)
+    rounded = f64(t(wide, torch.bfloat16))
+    g8, u8 = np.minimum(rounded[:, :48] + gb, limit), np.clip(rounded[:, 48:] + ub, -limit, limit)
+    close(ops.glu_clamped_bias(t(wide, torch.bfloat16), t(gb), t(ub), limit), g8 * P.sigmoid(1.702 * g8) * (u8 + 1), 8e-3,
+          "clamped gate, bfloat16")
     experts = 5
     up, dense = rng.standard_normal((rows, experts * ff)), rng.random((rows, experts)) * (rng.random((rows, experts)) < 0.5)
     want = (P.gelu_erf(up).reshape(rows, experts, ff) * dense[:, :, None]).reshape(rows, -1)
