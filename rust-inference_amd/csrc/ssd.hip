@@ -187,27 +187,31 @@ extern "C" int ri_ssd_scan(float* out, const float* xbc, int channels, int b_off
 // ------------------------------------------------------------------ the walk, a wavefront on 16 columns
 // States of up to 128 rows: a wavefront owns 16 columns of one (sequence, head), its lanes four slices of the rows of a
 // column each (8 columns and eight slices for states above 64 rows), the rows in registers; a token's sum over the rows is the lane's own sum (four partial sums, so that no
-// addition waits for the one before) and two exchanges between the lanes of a column.  A workgroup is one wavefront.
-// Tokens are staged in LDS in blocks of SSD_BLOCK (B, C, x, the step size and decay, z), the next block's loads asked
+// addition waits for the one before) and two exchanges between the lanes of a column.  A workgroup is four wavefronts
+// on columns of their own, which share the tokens staged in LDS in blocks of SSD_BLOCK (B, C, x, the step size and decay, z), the next block's loads asked
 // for before the block in work is computed.  The order of a token's additions is fixed by the sizes alone.
 #define SSD_BLOCK 8
+#define SSD_WAVES 4          // wavefronts of a workgroup: they share the staged tokens, each on columns of its own
 
 template <typename TA, int RPL, int SL>                       // RPL: rows a lane holds, a multiple of 4; SL: slices of rows, 4 or 8
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(64 * SSD_WAVES)
 ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int channels, int b_off, int c_off,
                      const TA* __restrict__ proj, int stride, int z_off, int dt_off, const float* __restrict__ dt_bias,
                      const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ state,
                      const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots, int heads, int groups, int n,
                      int vdim) {
-    constexpr int ROWS = SL * RPL, COLS = 64 / SL, TPP = 64 / COLS, PASSES = SSD_BLOCK / TPP;      // TPP: tokens whose x and z a pass fetches
+    // COLS: columns of a wavefront; NC: of the workgroup; TPP: tokens whose x and z one pass of the workgroup's threads fetches
+    constexpr int ROWS = SL * RPL, COLS = 64 / SL, NC = COLS * SSD_WAVES, THREADS = 64 * SSD_WAVES, TPP = THREADS / NC,
+                  PASSES = SSD_BLOCK / TPP;
     __shared__ __attribute__((aligned(16))) float bs[2][SSD_BLOCK][ROWS];
     __shared__ __attribute__((aligned(16))) float cs[2][SSD_BLOCK][ROWS];
-    __shared__ float xs[2][SSD_BLOCK][COLS];
-    __shared__ float zs[2][SSD_BLOCK][COLS];
+    __shared__ float xs[2][SSD_BLOCK][NC];
+    __shared__ float zs[2][SSD_BLOCK][NC];
     __shared__ float dts[2][SSD_BLOCK], decays[2][SSD_BLOCK];
-    const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int seq = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane % COLS, slice = lane / COLS, row0 = slice * RPL;
-    const int c = blockIdx.z * COLS + col;
+    const int wcol = wave * COLS + col;                       // the lane's column among the workgroup's
+    const int c = blockIdx.z * NC + wcol;
     const bool has_col = c < vdim;
     const int cc = has_col ? c : vdim - 1;                    // a column pulled back inside the head: loads are issued anyway
     const int group = h / (heads / groups), inner = heads * vdim;
@@ -217,43 +221,44 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
     for (int i = 0; i < RPL; ++i) st[i] = row0 + i < n ? sp[(size_t)(row0 + i) * vdim] : 0.f;
     const float neg_a = -expf(a_log[h]), skip = d_skip ? d_skip[h] : 0.f, bias = dt_bias ? dt_bias[h] : 0.f;
     const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
-    constexpr int PER = (2 * SSD_BLOCK * ROWS + 63) / 64;     // B and C elements of a block a lane stages
+    constexpr int PER = (2 * SSD_BLOCK * ROWS + THREADS - 1) / THREADS;     // B and C elements of a block a thread stages
+    const int vcol = min((int)blockIdx.z * NC + tid % NC, vdim - 1), vtok = tid / NC;      // the thread's place in a pass over x and z
 
     float pre_bc[PER], pre_x[PASSES], pre_z[PASSES], pre_raw = 0.f;
     auto fetch = [&](int tb) {                                // a block's loads, into registers
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int e = lane + i * 64;                      // (which, token, row)
+            const int e = tid + i * THREADS;                  // (which, token, row)
             const int r = e % ROWS, tt = (e / ROWS) % SSD_BLOCK, which = e / (ROWS * SSD_BLOCK);
             const int t = min(tb + tt, t1 - 1);
             pre_bc[i] = (r < n && which < 2) ? xbc[(size_t)t * channels + (which ? c_off : b_off) + group * n + r] : 0.f;
         }
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {                 // x and z of the block's tokens for this wavefront's columns
-            const int t = min(tb + ps * TPP + slice, t1 - 1);
-            pre_x[ps] = xbc[(size_t)t * channels + h * vdim + cc];
-            pre_z[ps] = to_f32(proj[(size_t)t * stride + z_off + h * vdim + cc]);
+            const int t = min(tb + ps * TPP + vtok, t1 - 1);
+            pre_x[ps] = xbc[(size_t)t * channels + h * vdim + vcol];
+            pre_z[ps] = to_f32(proj[(size_t)t * stride + z_off + h * vdim + vcol]);
         }
-        if (lane < SSD_BLOCK) pre_raw = to_f32(proj[(size_t)min(tb + lane, t1 - 1) * stride + dt_off + h]);
+        if (tid < SSD_BLOCK) pre_raw = to_f32(proj[(size_t)min(tb + tid, t1 - 1) * stride + dt_off + h]);
     };
     auto stage = [&](int buf) {                               // ... and from there into LDS
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int e = lane + i * 64;
+            const int e = tid + i * THREADS;
             const int r = e % ROWS, tt = (e / ROWS) % SSD_BLOCK, which = e / (ROWS * SSD_BLOCK);
             if (which == 0) bs[buf][tt][r] = pre_bc[i];
             else if (which == 1) cs[buf][tt][r] = pre_bc[i];
         }
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
-            xs[buf][ps * TPP + slice][col] = pre_x[ps];
-            zs[buf][ps * TPP + slice][col] = pre_z[ps];
+            xs[buf][ps * TPP + vtok][tid % NC] = pre_x[ps];
+            zs[buf][ps * TPP + vtok][tid % NC] = pre_z[ps];
         }
-        if (lane < SSD_BLOCK) {
+        if (tid < SSD_BLOCK) {
             const float raw = pre_raw + bias;
             const float dt = raw > 20.f ? raw : log1pf(expf(raw));       // softplus: beyond 20 it is its argument to the last bit
-            dts[buf][lane] = dt;
-            decays[buf][lane] = expf(neg_a * dt);
+            dts[buf][tid] = dt;
+            decays[buf][tid] = expf(neg_a * dt);
         }
     };
     if (t0 < t1) {
@@ -274,7 +279,7 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
             part[tt] = 0.f;
             if (tt < count) {
                 const float decay = decays[buf][tt];
-                const float dx = dts[buf][tt] * xs[buf][tt][col];
+                const float dx = dts[buf][tt] * xs[buf][tt][wcol];
                 float y0 = 0.f, y1 = 0.f, y2 = 0.f, y3 = 0.f;
 #pragma unroll
                 for (int i = 0; i < RPL; i += 4) {
@@ -295,8 +300,8 @@ ssd_scan_cols_kernel(float* __restrict__ out, const float* __restrict__ xbc, int
             y += __shfl_xor(y, 16, RI_WAVE);
             y += __shfl_xor(y, 32, RI_WAVE);
             if (tt < count && has_col && slice == 0) {
-                y += skip * xs[buf][tt][col];
-                const float z = zs[buf][tt][col];
+                y += skip * xs[buf][tt][wcol];
+                const float z = zs[buf][tt][wcol];
                 out[(size_t)(tb + tt) * inner + h * vdim + c] = y * (z / (1.f + expf(-z)));
             }
         }
@@ -323,12 +328,12 @@ extern "C" int ri_ssd_scan_cols(float* out, const float* xbc, int channels, int 
     RI_REQUIRE(z_off >= 0 && dt_off >= 0 && z_off + heads * vdim <= stride && dt_off + heads <= stride,
                "ssd_scan_cols: columns %d and %d of rows of %d", z_off, dt_off, stride);
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "ssd_scan_cols: dtype %d", act_dtype);
-    const int cols = n > 64 ? 8 : 16;
+    const int cols = (n > 64 ? 8 : 16) * SSD_WAVES;
     const dim3 grid(seqs, heads, (vdim + cols - 1) / cols);
     RI_REQUIRE(grid.z <= 65535, "ssd_scan_cols: heads of %d channels", vdim);
     hipStream_t s = (hipStream_t)stream;
 #define RI_GO(TA, RPL, SL)                                                                                              \
-    ssd_scan_cols_kernel<TA, RPL, SL><<<grid, 64, 0, s>>>(out, xbc, channels, b_off, c_off, (const TA*)proj, stride, z_off,  \
+    ssd_scan_cols_kernel<TA, RPL, SL><<<grid, 64 * SSD_WAVES, 0, s>>>(out, xbc, channels, b_off, c_off, (const TA*)proj, stride, z_off,  \
                                                       dt_off, dt_bias, a_log, d_skip, state, cu_seqlens, slots, heads,   \
                                                       groups, n, vdim)
 #define RI_BY_ROWS(TA)                                                                                                  \

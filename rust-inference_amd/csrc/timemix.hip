@@ -192,26 +192,30 @@ extern "C" int ri_timemix_scan(void* out, int out_stride, int out_off, float out
 // ------------------------------------------------------------------ the walk, a wavefront on 16 columns
 // Heads of up to 128: a wavefront owns 16 columns of one (sequence, head), its lanes four slices of the rows of a column
 // each (8 columns and eight slices for heads above 64: a token's walk over a lane's rows is what the wavefront waits for), the rows in registers; a token's sum over the rows is the lane's own sum (four partial sums, so that no addition
-// waits for the one before) and two exchanges between the lanes of a column.  A workgroup is one wavefront.  Tokens are
-// staged in LDS in blocks of TM_BLOCK (r, k, the decay, v), the next block's loads asked for before the block in work is
+// waits for the one before) and two exchanges between the lanes of a column.  A workgroup is four wavefronts on columns of
+// their own, which share the tokens staged in LDS in blocks of TM_BLOCK (r, k, the decay, v), the next block's loads asked for before the block in work is
 // computed.  The heads' results are written as they are, float32; the norm over a head and the gate are
 // heads_norm_gate's.
 #define TM_BLOCK 8
+#define TM_WAVES 4           // wavefronts of a workgroup: they share the staged tokens, each on columns of its own
 
 template <typename TA, int RPL, int SL>                       // RPL: rows a lane holds, a multiple of 4; SL: slices of rows, 4 or 8
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(64 * TM_WAVES)
 timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, const TA* __restrict__ k, const TA* __restrict__ v,
                          const float* __restrict__ z, const float* __restrict__ u,
                          float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
                          int heads, int dim) {
-    constexpr int ROWS = SL * RPL, COLS = 64 / SL, TPP = 64 / COLS, PASSES = TM_BLOCK / TPP;      // TPP: tokens whose v a pass of the wavefront fetches
+    // COLS: columns of a wavefront; NC: of the workgroup; TPP: tokens whose v one pass of the workgroup's threads fetches
+    constexpr int ROWS = SL * RPL, COLS = 64 / SL, NC = COLS * TM_WAVES, THREADS = 64 * TM_WAVES, TPP = THREADS / NC,
+                  PASSES = TM_BLOCK / TPP;
     __shared__ __attribute__((aligned(16))) float rs[2][TM_BLOCK][ROWS];
     __shared__ __attribute__((aligned(16))) float ks[2][TM_BLOCK][ROWS];
     __shared__ __attribute__((aligned(16))) float ws[2][TM_BLOCK][ROWS];
-    __shared__ float vs[2][TM_BLOCK][COLS];
-    const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    __shared__ float vs[2][TM_BLOCK][NC];
+    const int seq = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane % COLS, slice = lane / COLS, row0 = slice * RPL;
-    const int c = blockIdx.z * COLS + col;
+    const int wcol = wave * COLS + col;                       // the lane's column among the workgroup's
+    const int c = blockIdx.z * NC + wcol;
     const bool has_col = c < dim;
     const int cc = has_col ? c : dim - 1;                     // a column pulled back inside the head: loads are issued anyway
     const int width = heads * dim;
@@ -223,13 +227,14 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
         ub[i] = row0 + i < dim ? u[h * dim + row0 + i] : 0.f;
     }
     const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
-    constexpr int PER = (TM_BLOCK * ROWS + 63) / 64;          // elements of each of r, k and the decay that a lane stages
+    constexpr int PER = (TM_BLOCK * ROWS + THREADS - 1) / THREADS;      // elements of each of r, k and the decay that a thread stages
+    const int vcol = min((int)blockIdx.z * NC + tid % NC, dim - 1), vtok = tid / NC;      // the thread's place in a pass over v
 
     float pre_r[PER], pre_k[PER], pre_w[PER], pre_v[PASSES];
     auto fetch = [&](int tb) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int e = lane + i * 64;
+            const int e = tid + i * THREADS;
             const int row = e % ROWS, tt = e / ROWS;
             const bool in = row < dim && tt < TM_BLOCK;
             const size_t at = (size_t)min(tb + tt, t1 - 1) * width + (size_t)h * dim + (in ? row : 0);
@@ -239,12 +244,12 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
         }
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps)
-            pre_v[ps] = to_f32(v[(size_t)min(tb + ps * TPP + slice, t1 - 1) * width + (size_t)h * dim + cc]);
+            pre_v[ps] = to_f32(v[(size_t)min(tb + ps * TPP + vtok, t1 - 1) * width + (size_t)h * dim + vcol]);
     };
     auto stage = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int e = lane + i * 64;
+            const int e = tid + i * THREADS;
             const int row = e % ROWS, tt = e / ROWS;
             if (tt < TM_BLOCK) {
                 rs[buf][tt][row] = pre_r[i];
@@ -253,7 +258,7 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
             }
         }
 #pragma unroll
-        for (int ps = 0; ps < PASSES; ++ps) vs[buf][ps * TPP + slice][col] = pre_v[ps];
+        for (int ps = 0; ps < PASSES; ++ps) vs[buf][ps * TPP + vtok][tid % NC] = pre_v[ps];
     };
     if (t0 < t1) {
         fetch(t0);
@@ -270,7 +275,7 @@ timemix_scan_cols_kernel(float* __restrict__ out, const TA* __restrict__ r, cons
         for (int tt = 0; tt < TM_BLOCK; ++tt) {
             part[tt] = 0.f;
             if (tt < count) {
-                const float vc = vs[buf][tt][col];
+                const float vc = vs[buf][tt][wcol];
                 float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
                 for (int i = 0; i < RPL; i += 4) {
@@ -341,14 +346,14 @@ extern "C" int ri_timemix_scan_cols(void* out, int out_stride, int out_off, floa
                "timemix_scan_cols: %d tokens of %d sequences, %d heads of %d", tokens, seqs, heads, dim);
     RI_REQUIRE(out_off >= 0 && out_off + heads * dim <= out_stride, "timemix_scan_cols: column %d of rows of %d", out_off, out_stride);
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "timemix_scan_cols: dtype %d", act_dtype);
-    const int cols = dim > 64 ? 8 : 16;
+    const int cols = (dim > 64 ? 8 : 16) * TM_WAVES;
     const dim3 grid(seqs, heads, (dim + cols - 1) / cols);
     hipStream_t s = (hipStream_t)stream;
     const long total = (long)tokens * heads * dim;
     RI_REQUIRE((total + 255) / 256 <= 2147483647L, "timemix_scan_cols: %ld decays exceed one launch", total);
     timemix_decay_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(z, w0, total, heads * dim);
 #define RI_GO(TA, ROWS, SL)                                                                                             \
-    timemix_scan_cols_kernel<TA, ROWS, SL><<<grid, 64, 0, s>>>(o, (const TA*)r, (const TA*)k, (const TA*)v, z, u, state,  \
+    timemix_scan_cols_kernel<TA, ROWS, SL><<<grid, 64 * TM_WAVES, 0, s>>>(o, (const TA*)r, (const TA*)k, (const TA*)v, z, u, state,  \
                                                            cu_seqlens, slots, heads, dim)
 #define RI_BY_ROWS(TA)                                                                                                  \
     if (dim <= 16) RI_GO(TA, 4, 4); else if (dim <= 32) RI_GO(TA, 8, 4); else if (dim <= 64) RI_GO(TA, 16, 4); else RI_GO(TA, 16, 8)

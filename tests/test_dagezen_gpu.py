@@ -393,7 +393,7 @@ def drawn_config(seed):
         elif kind == "par":
             kv = pick([1, 2, 3, 4])
             mixer = par(kv * pick([1, 2, 4]), kv, pick([8, 16, 24, 32, 48, 64]), float(rng.uniform(0.05, 0.4)),
-                        pick([None, 1, 7, 31, 32, 33, 50, 100, 136]), pick([1, 2, 3, 5]), pick([8, 24, 32, 48, 64, 100]),
+                        pick([None, 1, 7, 31, 32, 33, 50, 100, 150]), pick([1, 2, 3, 5]), pick([8, 24, 32, 48, 64, 100]),
                         float(rng.uniform(0.3, 1.5)), float(rng.uniform(0.3, 1.5)), rank=pick([1, 8, 16]))
         else:
             groups = pick([1, 2, 3])
