@@ -413,12 +413,13 @@ int ri_head_products(void* out, int out_dtype, int out_stride, int out_off, int 
                      int x_stride, int x_off, int x_head, const void* w, int w_dtype, const void* gates, int g_stride,
                      int g_off, float scale, int tokens, int heads, int k, int n, int extra, void* stream);
 // The attention over the cached latent on the matrix cores (latent_mfma.hip): bfloat16, pages of 32, (key_dim, rank) one of
-// (576, 512), (288, 256), (160, 128).
+// (576, 512), (288, 256), (160, 128).  chunks > 1: a token's pages in chunks of chunk_pages that run side by side, joined by a
+// second launch; partial: float32 workspace [tokens][heads][chunks][rank + 2].
 int ri_latent_attention_mfma_fits(int key_dim, int rank, int page_size);
 int ri_latent_attention_mfma(void* out, const void* q, int q_stride, const void* k_pages, const void* v_pages,
                              const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table, int table_width,
                              int tokens, int heads, int key_dim, int rank, int page_size, float scale, const float* sinks,
-                             void* stream);
+                             float* partial, int chunks, int chunk_pages, void* stream);
 
 // ---- windowed attention whose heads talk (talking_attention.hip)
 int ri_whole_norm_kv_write(void* proj, int act_dtype, int stride, int q_off, int k_off, const float* q_gain,

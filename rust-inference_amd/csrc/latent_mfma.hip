@@ -9,6 +9,8 @@
 // how the value product wants its weights: no exchange between lanes.  A sink per head joins the sum once at the end.
 // Scores, maxima, sums and the accumulators are float32; the weights are rounded to bfloat16 for the value product, as
 // in this library's other matrix-core attention.  A token's sums run over its pages in order, whatever else the step holds.
+// A step of few tokens cuts a token's pages into chunks that wavefronts walk side by side; each leaves its maximum, its sum
+// and its sums of values, and a second kernel joins them in the chunks' order.
 #include "api.h"
 #include "common.h"
 
@@ -30,11 +32,13 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict_
                              const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                              const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
                              const int32_t* __restrict__ page_table, int table_width, int tokens, int heads, int tiles,
-                             float scale_log2, const float* __restrict__ sinks) {
+                             float scale_log2, const float* __restrict__ sinks, float* __restrict__ partial, int chunks,
+                             int chunk_pages) {
     constexpr int DK = 32 * KS, RANK = 16 * VT;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int pair = blockIdx.x * LM_WAVES + wave;            // (token, tile of 16 heads)
-    if (pair >= tokens * tiles) return;
+    const int unit = blockIdx.x * LM_WAVES + wave;            // (token, tile of 16 heads, chunk of pages)
+    if (unit >= tokens * tiles * chunks) return;
+    const int pair = unit / chunks, chunk = unit % chunks;
     // (long prompts first: the workgroups launched last are the short ones)
     const int t = tokens - 1 - pair / tiles, tile = pair % tiles;
     const int col = lane & 15, g = lane >> 4;
@@ -53,7 +57,8 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict_
     float m = -INFINITY, l = 0.f;
     const int key_row = 8 * (col >> 2) + (col & 3);           // the key this lane's operand row holds in the first half page
 
-    for (int page = 0; page <= qpos / LM_PAGE; ++page) {
+    const int page_end = chunks > 1 ? min(qpos / LM_PAGE + 1, (chunk + 1) * chunk_pages) : qpos / LM_PAGE + 1;
+    for (int page = chunks > 1 ? chunk * chunk_pages : 0; page < page_end; ++page) {
         const long phys = table[page];
         const bf16_t* kp = k_pages + phys * LM_PAGE * (long)DK + (long)key_row * DK + 8 * g;
         lm_floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -99,6 +104,18 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict_
     }
     l += __shfl_xor(l, 16, RI_WAVE);                          // a column's sum over its four lanes
     l += __shfl_xor(l, 32, RI_WAVE);
+    if (chunks > 1) {
+        // a chunk's share: its maximum, its sum and its sums of values as they are, for the join (a chunk without pages: -inf, 0, 0)
+        if (head < heads) {
+            float* pp = partial + (((size_t)t * heads + head) * chunks + chunk) * (RANK + 2);
+            if (g == 0) { pp[0] = m; pp[1] = l; }
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) pp[2 + vt * 16 + 4 * g + i] = o[vt][i];
+        }
+        return;
+    }
     if (sinks) l += exp2f(sinks[hq] * 1.4426950408889634f - m);
     const float inv = 1.0f / l;
     if (head < heads) {
@@ -113,6 +130,25 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict_
     }
 }
 
+// The chunks of a token's pages, joined: the largest maximum, every chunk's sums scaled to it, the sink, the division.
+__global__ void __launch_bounds__(256)
+latent_attention_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial, const float* __restrict__ sinks,
+                             int heads, int chunks, int rank) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    const float* pp = partial + ((size_t)t * heads + h) * chunks * (rank + 2);
+    float m = -INFINITY;
+    for (int c = 0; c < chunks; ++c) m = fmaxf(m, pp[(size_t)c * (rank + 2)]);
+    float l = 0.f;
+    for (int c = 0; c < chunks; ++c) l += pp[(size_t)c * (rank + 2) + 1] * exp2f(pp[(size_t)c * (rank + 2)] - m);
+    if (sinks) l += exp2f(sinks[h] * 1.4426950408889634f - m);
+    const float inv = 1.0f / l;
+    for (int d = threadIdx.x; d < rank; d += 256) {
+        float a = 0.f;
+        for (int c = 0; c < chunks; ++c) a += pp[(size_t)c * (rank + 2) + 2 + d] * exp2f(pp[(size_t)c * (rank + 2)] - m);
+        out[((size_t)t * heads + h) * rank + d] = f32_to_bf16(a * inv);
+    }
+}
+
 extern "C" int ri_latent_attention_mfma_fits(int key_dim, int rank, int page_size) {
     return page_size == LM_PAGE && ((key_dim == 576 && rank == 512) || (key_dim == 288 && rank == 256) || (key_dim == 160 && rank == 128));
 }
@@ -122,15 +158,17 @@ extern "C" int ri_latent_attention_mfma_fits(int key_dim, int rank, int page_siz
 extern "C" int ri_latent_attention_mfma(void* out, const void* q, int q_stride, const void* k_pages, const void* v_pages,
                                         const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
                                         int table_width, int tokens, int heads, int key_dim, int rank, int page_size, float scale,
-                                        const float* sinks, void* stream) {
+                                        const float* sinks, float* partial, int chunks, int chunk_pages, void* stream) {
     RI_REQUIRE(tokens > 0 && heads > 0 && ri_latent_attention_mfma_fits(key_dim, rank, page_size),
                "latent_attention_mfma: %d tokens, %d heads, keys of %d, values of %d, pages of %d", tokens, heads, key_dim, rank, page_size);
     RI_REQUIRE(q_stride >= heads * key_dim && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 &&
                (uintptr_t)v_pages % 16 == 0 && (uintptr_t)out % 8 == 0, "latent_attention_mfma: rows of %d for %d heads of %d, or a buffer that is not aligned",
                q_stride, heads, key_dim);
     RI_REQUIRE(scale > 0.f && table_width > 0, "latent_attention_mfma: scale %g", (double)scale);
+    RI_REQUIRE(chunks >= 1 && (chunks == 1 || (partial && chunk_pages >= 1)) && heads <= 65535,
+               "latent_attention_mfma: %d chunks of %d pages", chunks, chunk_pages);
     const int tiles = (heads + 15) / 16;
-    const long pairs = (long)tokens * tiles;
+    const long pairs = (long)tokens * tiles * chunks;
     RI_REQUIRE((pairs + LM_WAVES - 1) / LM_WAVES <= 2147483647L, "latent_attention_mfma: %ld tiles exceed one launch", pairs);
     const unsigned blocks = (unsigned)((pairs + LM_WAVES - 1) / LM_WAVES);
     const float scale_log2 = scale * 1.4426950408889634f;
@@ -139,9 +177,12 @@ extern "C" int ri_latent_attention_mfma(void* out, const void* q, int q_stride, 
     latent_attention_mfma_kernel<KS, VT><<<blocks, 64 * LM_WAVES, 0, s>>>((bf16_t*)out, (const bf16_t*)q, q_stride,     \
                                                                           (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
                                                                           tok_pos, tok_seq, page_table, table_width, tokens, \
-                                                                          heads, tiles, scale_log2, sinks)
+                                                                          heads, tiles, scale_log2, sinks, partial, chunks, \
+                                                                          chunk_pages)
     if (key_dim == 576) RI_GO(18, 32); else if (key_dim == 288) RI_GO(9, 16); else RI_GO(5, 8);
 #undef RI_GO
+    if (chunks > 1)
+        latent_attention_join_kernel<<<dim3(tokens, heads), 256, 0, s>>>((bf16_t*)out, partial, sinks, heads, chunks, rank);
     RI_LAUNCH_CHECK("latent_attention_mfma");
     return 0;
 }

@@ -136,7 +136,7 @@ _SIGNATURES = {
                           c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_latent_attention_mfma_fits": [c_int, c_int, c_int],
     "ri_latent_attention_mfma": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                 c_int, c_int, c_int, c_float, c_void_p, c_void_p],
+                                 c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_head_products": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
                          c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_whole_norm_kv_write": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
@@ -1343,20 +1343,31 @@ def latent_attention_mfma_fits(dtype, key_dim: int, rank: int, page_size: int) -
     return dtype == torch.bfloat16 and bool(_get("ri_latent_attention_mfma_fits")(key_dim, rank, page_size))
 
 
-def latent_attention_mfma(q, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, scale: float, sinks) -> torch.Tensor:
+def latent_attention_mfma(q, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, scale: float, sinks,
+                          max_len: int = 0) -> torch.Tensor:
     """bfloat16 ``[T, heads * rank]``: causal attention on the matrix cores of every new token's ``heads`` query rows (``q [T,
     heads * key_dim]``) over its sequence's single key/value head (``k_pages [pages, 1, 32, key_dim]``, ``v_pages [pages, 1, rank,
-    32]``), with a sink per head in the softmax's denominator (or None)."""
+    32]``), with a sink per head in the softmax's denominator (or None).  ``max_len``: a bound on the sequences' lengths; given, a
+    step of few tokens cuts every token's pages into chunks that run side by side and are joined by a second launch."""
     tokens = q.shape[0]
     key_dim, rank, page = k_pages.shape[3], v_pages.shape[2], k_pages.shape[2]
     if k_pages.shape[1] != 1 or v_pages.shape[1] != 1 or v_pages.shape[3] != page or q.shape[1] != heads * key_dim:
         raise ShapeError(f"latent_attention_mfma: q {list(q.shape)}, key pages {list(k_pages.shape)}, value pages {list(v_pages.shape)}")
     out = torch.empty((tokens, heads * rank), dtype=torch.bfloat16, device=q.device)
+    chunks, chunk_pages, partial = 1, 0, None
+    units = tokens * -(-heads // 16)
+    if max_len and units < 256:                      # fewer wavefronts than half the machine's SIMDs: chunks of pages side by side
+        pages = -(-int(max_len) // page)
+        chunks = max(1, min(pages, 512 // units, 64))
+        chunk_pages = -(-pages // chunks)
+        chunks = -(-pages // chunk_pages)
+        if chunks > 1:
+            partial = torch.empty((tokens, heads, chunks, rank + 2), dtype=torch.float32, device=q.device)
     _call("ri_latent_attention_mfma", _dev(out, "out"), _dev(q, "q", torch.bfloat16), q.shape[1],
           _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
           _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], tokens, heads, key_dim, rank, page, float(scale),
-          _opt(sinks, "sinks", torch.float32, (heads,)), _stream())
+          _opt(sinks, "sinks", torch.float32, (heads,)), _opt(partial, "partial"), chunks, chunk_pages, _stream())
     return out
 
 

@@ -97,13 +97,12 @@ class LatentAttention(Mixer):
             else:
                 raise ConfigError("a latent attention without unrotated elements has no kernel")
         with profiler.section(profiler.ATTENTION):
-            if (not ctx.is_decode and not rt.invariant
-                    and ops.latent_attention_mfma_fits(q.dtype, self.rank + self.rot, self.rank, store.page_size)):
-                # prompts at the sizes the matrix cores take: a wavefront on 16 heads of a token walks the token's pages
-                # (for single tokens that walk is too long for the two wavefronts a sequence has: 319 us for 1,024 keys
-                # where the general kernel, a workgroup a head, takes 106)
+            if not rt.invariant and ops.latent_attention_mfma_fits(q.dtype, self.rank + self.rot, self.rank, store.page_size):
+                # the sizes the matrix cores take: a wavefront on 16 heads of a token walks the token's pages; a step of few
+                # tokens cuts the pages into chunks side by side (one walk of 1,024 keys by the two wavefronts a sequence has
+                # takes 319 us, the general kernel 106)
                 o = ops.latent_attention_mfma(q, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
-                                              self.scale, self.sink)
+                                              self.scale, self.sink, ctx.max_len if ctx.is_decode else 0)
             else:
                 o = ops.attention(q, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads, 1,
                                   self.rank + self.rot, None, self.scale, sinks=self.sink)

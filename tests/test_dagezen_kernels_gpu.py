@@ -319,6 +319,9 @@ def test_latent_attention_on_the_matrix_cores_is_the_general_kernel(ops, heads):
         want = ops.attention(q, k_pages, v_pages, tok_pos, tok_seq, table, heads, 1, dk, None, 0.11, sinks=sink)
         got = ops.latent_attention_mfma(q, k_pages, v_pages, tok_pos, tok_seq, table, heads, 0.11, sink)
         close(got, f64(want), 1.2e-2, "matrix cores against the general kernel")
+        for bound in (101, 128, 1024):                    # chunks of one page, of one page with more room than pages, of eight
+            got = ops.latent_attention_mfma(q, k_pages, v_pages, tok_pos, tok_seq, table, heads, 0.11, sink, bound)
+            close(got, f64(want), 1.2e-2, f"in chunks, sequences of up to {bound}")
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, window", [(8, 2, 32, 40), (16, 16, 32, None), (8, 1, 64, 33)])
