@@ -25,6 +25,7 @@ union LmFrag {
 
 #define LM_PAGE 32
 #define LM_WAVES 4
+#define LM_MAX_CHUNKS 64
 
 template <int KS, int VT>
 __global__ void __launch_bounds__(64 * LM_WAVES)
@@ -134,17 +135,34 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict_
 __global__ void __launch_bounds__(256)
 latent_attention_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial, const float* __restrict__ sinks,
                              int heads, int chunks, int rank) {
-    const int t = blockIdx.x, h = blockIdx.y;
+    __shared__ float ms[LM_MAX_CHUNKS], ws[LM_MAX_CHUNKS], ls[LM_MAX_CHUNKS];
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const float* pp = partial + ((size_t)t * heads + h) * chunks * (rank + 2);
+    if (tid < chunks) {
+        ms[tid] = pp[(size_t)tid * (rank + 2)];
+        ls[tid] = pp[(size_t)tid * (rank + 2) + 1];
+    }
+    __syncthreads();
     float m = -INFINITY;
-    for (int c = 0; c < chunks; ++c) m = fmaxf(m, pp[(size_t)c * (rank + 2)]);
+    for (int c = 0; c < chunks; ++c) m = fmaxf(m, ms[c]);
+    if (tid < chunks) ws[tid] = exp2f(ms[tid] - m);           // a chunk's factor, once
+    __syncthreads();
     float l = 0.f;
-    for (int c = 0; c < chunks; ++c) l += pp[(size_t)c * (rank + 2) + 1] * exp2f(pp[(size_t)c * (rank + 2)] - m);
+    for (int c = 0; c < chunks; ++c) l += ls[c] * ws[c];
     if (sinks) l += exp2f(sinks[h] * 1.4426950408889634f - m);
     const float inv = 1.0f / l;
-    for (int d = threadIdx.x; d < rank; d += 256) {
+    for (int d = tid; d < rank; d += 256) {
+        const float* col = pp + 2 + d;
         float a = 0.f;
-        for (int c = 0; c < chunks; ++c) a += pp[(size_t)c * (rank + 2) + 2 + d] * exp2f(pp[(size_t)c * (rank + 2)] - m);
+        int c = 0;
+        for (; c + 8 <= chunks; c += 8) {                     // eight loads asked for before the first is used
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = col[(size_t)(c + i) * (rank + 2)];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a += v[i] * ws[c + i];
+        }
+        for (; c < chunks; ++c) a += col[(size_t)c * (rank + 2)] * ws[c];
         out[((size_t)t * heads + h) * rank + d] = f32_to_bf16(a * inv);
     }
 }
@@ -165,7 +183,7 @@ extern "C" int ri_latent_attention_mfma(void* out, const void* q, int q_stride, 
                (uintptr_t)v_pages % 16 == 0 && (uintptr_t)out % 8 == 0, "latent_attention_mfma: rows of %d for %d heads of %d, or a buffer that is not aligned",
                q_stride, heads, key_dim);
     RI_REQUIRE(scale > 0.f && table_width > 0, "latent_attention_mfma: scale %g", (double)scale);
-    RI_REQUIRE(chunks >= 1 && (chunks == 1 || (partial && chunk_pages >= 1)) && heads <= 65535,
+    RI_REQUIRE(chunks >= 1 && chunks <= LM_MAX_CHUNKS && (chunks == 1 || (partial && chunk_pages >= 1)) && heads <= 65535,
                "latent_attention_mfma: %d chunks of %d pages", chunks, chunk_pages);
     const int tiles = (heads + 15) / 16;
     const long pairs = (long)tokens * tiles * chunks;

@@ -193,11 +193,20 @@ glu_clamped_bias_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restric
         u[2 * e] = __uint_as_float(uw[e] << 16);
         u[2 * e + 1] = __uint_as_float(uw[e] & 0xFFFF0000u);
     }
+    float bg[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, bu[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (b_gate) {
+        const float4 x = *reinterpret_cast<const float4*>(b_gate + i), y = *reinterpret_cast<const float4*>(b_gate + i + 4);
+        bg[0] = x.x; bg[1] = x.y; bg[2] = x.z; bg[3] = x.w; bg[4] = y.x; bg[5] = y.y; bg[6] = y.z; bg[7] = y.w;
+    }
+    if (b_up) {
+        const float4 x = *reinterpret_cast<const float4*>(b_up + i), y = *reinterpret_cast<const float4*>(b_up + i + 4);
+        bu[0] = x.x; bu[1] = x.y; bu[2] = x.z; bu[3] = x.w; bu[4] = y.x; bu[5] = y.y; bu[6] = y.z; bu[7] = y.w;
+    }
     uint32_t o[4];
     float a[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        float gv = g[e] + (b_gate ? b_gate[i + e] : 0.f), uv = u[e] + (b_up ? b_up[i + e] : 0.f);
+        float gv = g[e] + bg[e], uv = u[e] + bu[e];
         gv = fminf(gv, limit);
         uv = fminf(fmaxf(uv, -limit), limit);
         a[e] = gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f);
@@ -219,7 +228,8 @@ extern "C" int ri_glu_clamped_bias(void* out, const void* gu, int dtype, const f
         if (dtype == RI_F32)
             glu_clamped_bias_kernel<float><<<grid, 256, 0, s>>>((float*)out + (size_t)r0 * ff, (const float*)gu + (size_t)r0 * 2 * ff,
                                                                b_gate, b_up, limit, ff);
-        else if (ff % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0)
+        else if (ff % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)b_gate % 16 == 0 &&
+                 (uintptr_t)b_up % 16 == 0)
             glu_clamped_bias_bf16x8_kernel<<<dim3((ff / 8 + 255) / 256, n), 256, 0, s>>>(
                 (bf16_t*)out + (size_t)r0 * ff, (const bf16_t*)gu + (size_t)r0 * 2 * ff, b_gate, b_up, limit, ff);
         else
