@@ -156,7 +156,8 @@ head_products_kernel(TO* __restrict__ out, int out_stride, int out_off, int out_
 extern "C" int ri_head_products(void* out, int out_dtype, int out_stride, int out_off, int out_head, const void* x, int x_dtype,
                                 int x_stride, int x_off, int x_head, const void* w, int w_dtype, const void* gates, int g_stride,
                                 int g_off, float scale, int tokens, int heads, int k, int n, int extra, void* stream) {
-    RI_REQUIRE(tokens > 0 && heads > 0 && heads <= 65535 && k > 0 && n > 0 && extra >= 0,
+    // k = n = 0: no product, the copied elements alone (with the head's gate and the scale); w is not read
+    RI_REQUIRE(tokens > 0 && heads > 0 && heads <= 65535 && extra >= 0 && ((k > 0 && n > 0) || (k == 0 && n == 0 && extra > 0)),
                "head_products: %d tokens, %d heads of %d x %d (+%d)", tokens, heads, k, n, extra);
     RI_REQUIRE(x_off >= 0 && x_head >= k + extra && x_off + (long)(heads - 1) * x_head + k + extra <= x_stride,
                "head_products: heads of %d at column %d of rows of %d", x_head, x_off, x_stride);

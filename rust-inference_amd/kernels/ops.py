@@ -1390,6 +1390,47 @@ def head_products(x, x_off: int, x_head: int, w, heads: int, k: int, n: int, ext
     return out
 
 
+def head_gate_copy(out, out_off: int, out_head: int, x, x_off: int, x_head: int, heads: int, width: int, gates=None,
+                   g_off: int = 0, scale: float = 1.0) -> None:
+    """``out[t, out_off + h * out_head + (0..width)] = scale * sigmoid(gates[t, g_off + h]) * x[t, x_off + h * x_head + (0..width)]``:
+    the copying half of ``head_products`` alone (no matrices)."""
+    tokens = x.shape[0]
+    if out.shape[0] != tokens or (gates is not None and (gates.shape[0] != tokens or gates.dtype != x.dtype)):
+        raise ShapeError(f"head_gate_copy: out {list(out.shape)}, x {list(x.shape)}")
+    _call("ri_head_products", _dev(out, "out"), code(out.dtype), out.shape[1], int(out_off), int(out_head), _dev(x, "x"),
+          code(x.dtype), x.shape[1], int(x_off), int(x_head), _dev(x, "x"), code(x.dtype), _opt(gates, "gates"),
+          gates.shape[1] if gates is not None else 0, int(g_off), float(scale), tokens, heads, 0, 0, int(width), _stream())
+
+
+BATCHED_HEAD_PRODUCTS_FROM = 128       # tokens of a step from which the products per head go to the library
+
+
+def head_products_batched(x, x_off: int, x_head: int, w, heads: int, k: int, n: int, extra: int = 0, gates=None,
+                          g_off: int = 0) -> torch.Tensor:
+    """What ``head_products`` gives for bfloat16 rows, with the products as one batched product of the library over the
+    heads (float32 sums, rounded once); the copied elements and the gates go through ``head_gate_copy``.  For steps of
+    many tokens: the library's product runs on the matrix cores, ``head_products`` on the vector units."""
+    tokens = x.shape[0]
+    if tuple(w.shape) != (heads, k, n) or x.dim() != 2 or x.stride(1) != 1 or not w.is_contiguous():
+        raise ShapeError(f"head_products_batched: matrices {list(w.shape)} for {heads} heads of {k} x {n}, rows {list(x.shape)}")
+    if x_off < 0 or x_head < k + extra or x_off + (heads - 1) * x_head + k + extra > x.shape[1]:
+        raise ShapeError(f"head_products_batched: heads of {x_head} at column {x_off} of rows of {x.shape[1]}")
+    out_head = n + extra
+    out = torch.empty((tokens, heads * out_head), dtype=x.dtype, device=x.device)
+    xv = x.as_strided((heads, tokens, k), (x_head, x.stride(0), 1), x.storage_offset() + x_off)
+    if gates is None:
+        torch.bmm(xv, w, out=out.as_strided((heads, tokens, n), (out_head, out.stride(0), 1)))
+        if extra:
+            head_gate_copy(out, n, out_head, x, x_off + k, x_head, heads, extra)
+        return out
+    plain = torch.empty_like(out)
+    torch.bmm(xv, w, out=plain.as_strided((heads, tokens, n), (out_head, plain.stride(0), 1)))
+    if extra:
+        head_gate_copy(plain, n, out_head, x, x_off + k, x_head, heads, extra)
+    head_gate_copy(out, 0, out_head, plain, 0, out_head, heads, out_head, gates=gates, g_off=g_off)
+    return out
+
+
 # ---------------------------------------------------------------- windowed attention whose heads talk
 def whole_norm_kv_write(proj, q_off: int, k_off: int, q_gain, k_gain, eps: float, tok_pos, tok_seq, page_table, k_pages,
                         v_pages, heads: int, kv_heads: int, dim: int) -> None:

@@ -92,7 +92,13 @@ class LatentAttention(Mixer):
         with profiler.section(profiler.QK_NORM_ROPE_APPEND):
             ops.latent_prepare(proj, 0, kv_at, self.c_gain, self.eps, self.inv_freq, ctx.tok_pos, ctx.tok_seq, page_table,
                                store.k_pages, store.v_pages, self.heads, self.dim, self.rot, self.rank)
-            if self.dim:
+            # steps of many bfloat16 tokens: the products per head as one batched product of the library
+            batched = (not rt.invariant and proj.dtype == torch.bfloat16 and self.w_uv.dtype == torch.bfloat16
+                       and proj.shape[0] >= ops.BATCHED_HEAD_PRODUCTS_FROM)
+            if self.dim and batched:
+                q = ops.head_products_batched(proj, 0, self.dim + self.rot, self.w_uk, self.heads, self.dim, self.rank,
+                                              extra=self.rot)
+            elif self.dim:
                 q = ops.head_products(proj, 0, self.dim + self.rot, self.w_uk, self.heads, self.dim, self.rank, extra=self.rot)
             else:
                 raise ConfigError("a latent attention without unrotated elements has no kernel")
@@ -106,7 +112,11 @@ class LatentAttention(Mixer):
             else:
                 o = ops.attention(q, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads, 1,
                                   self.rank + self.rot, None, self.scale, sinks=self.sink)
-            heads = ops.head_products(o, 0, self.rank, self.w_uv, self.heads, self.rank, self.vdim,
-                                      gates=proj if self.gate else None, g_off=kv_at + self.rank + self.rot)
+            if batched and o.dtype == torch.bfloat16:
+                heads = ops.head_products_batched(o, 0, self.rank, self.w_uv, self.heads, self.rank, self.vdim,
+                                                  gates=proj if self.gate else None, g_off=kv_at + self.rank + self.rot)
+            else:
+                heads = ops.head_products(o, 0, self.rank, self.w_uv, self.heads, self.rank, self.vdim,
+                                          gates=proj if self.gate else None, g_off=kv_at + self.rank + self.rot)
         with profiler.section(profiler.OUT_PROJECTION):
             return rt.linear_packed(heads, self.w_o, out_dtype=torch.float32, parts_ok=True)

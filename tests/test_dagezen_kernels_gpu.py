@@ -302,6 +302,33 @@ def test_state_space_mixer_through_every_cut(ops, heads, vdim, n, groups, taps, 
         close(got, np.concatenate(want), 3e-5, f"state-space mixer, step {counts}")
 
 
+# ---------------------------------------------------------------- the products per head through the library
+@pytest.mark.parametrize("heads, k, n, extra, gated", [(3, 24, 40, 6, False), (5, 40, 12, 0, True), (2, 16, 16, 10, True)])
+def test_batched_head_products_are_the_products_per_head(ops, heads, k, n, extra, gated):
+    """bfloat16 rows with the heads somewhere inside a wider row, columns in front and behind: the batched product with the
+    copied elements and a gate a head against the sums written out in float64, and beside the kernel that does it alone."""
+    rng = np.random.default_rng(heads)
+    tokens, x_off, x_head = 37, 5, k + extra + 3
+    stride = x_off + heads * x_head + heads + 4
+    x = t(rng.standard_normal((tokens, stride)), torch.bfloat16)
+    w = t(rng.standard_normal((heads, k, n)) / 4, torch.bfloat16)
+    g_off = x_off + heads * x_head + 2
+    got = ops.head_products_batched(x, x_off, x_head, w, heads, k, n, extra=extra, gates=x if gated else None, g_off=g_off)
+    alone = ops.head_products(x, x_off, x_head, w, heads, k, n, extra=extra, gates=x if gated else None, g_off=g_off)
+    xs, ws = f64(x), f64(w)
+    want = np.zeros((tokens, heads, n + extra))
+    for h in range(heads):
+        rows = xs[:, x_off + h * x_head: x_off + (h + 1) * x_head]
+        want[:, h, :n] = rows[:, :k] @ ws[h]
+        want[:, h, n:] = rows[:, k:k + extra]
+        if gated:
+            want[:, h] *= (1 / (1 + np.exp(-xs[:, g_off + h])))[:, None]
+    want = want.reshape(tokens, -1)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == want.shape
+    close(got, want, 1.2e-2, "batched products per head")          # two roundings to bfloat16 with a gate, one without
+    close(alone, want, 6e-3, "products per head")
+
+
 # ---------------------------------------------------------------- the latent attention on the matrix cores
 @pytest.mark.parametrize("heads", [3, 20])
 def test_latent_attention_on_the_matrix_cores_is_the_general_kernel(ops, heads):
