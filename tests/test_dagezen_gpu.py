@@ -38,7 +38,12 @@ D_B = model([layer(latent(4, 64, 32, 64, 256, 0.08, 1000000.0), dense(256, 3.0))
 D_C = model([layer(ssm(3, 16, 1, 3, 5, 3), dense(40, 2.0)), layer(par(4, 4, 32, 0.15, 32, 1, 40, 1.0, 0.5), moe(1, 1, 56)),
              layer(latent(2, 30, 2, 8, 20, 0.2, 100.0), moe(6, 4, 16)), layer(par(2, 1, 8, 0.5, 1, 4, 16, 0.5, 1.5), dense(96, 1.0))],
             vocab=157, width=64, eps=1e-5, alpha=3.0, cap=30.0)
-CONFIGS = {"A": D_A, "B": D_B, "C": D_C}
+# Sizes that 16-byte loads do not divide: a width of 100, heads of 12 and 20, a latent of 36 with six rotated elements,
+# feed-forwards of 52 and 28, a window over more than a page beside one over everything a test sends.
+D_D = model([layer(latent(5, 12, 6, 20, 36, 0.2), dense(52, 1.5)), layer(par(6, 3, 20, 0.2, 41, 3, 12, 0.8, 1.1, rank=5), moe(5, 2, 28)),
+             layer(ssm(6, 12, 20, 3, 4, 3), dense(100, 3.0)), layer(par(5, 5, 12, 0.3, 500, 5, 20, 1.0, 1.0, rank=3), None)],
+            vocab=333, width=100, eps=1e-5, alpha=2.6, cap=20.0)
+CONFIGS = {"A": D_A, "B": D_B, "C": D_C, "D": D_D}
 
 
 def sharpen(folder):
@@ -161,7 +166,7 @@ def in_portions(requests, sizes):
     return steps
 
 
-LENGTHS = {"A": [70, 3, 131], "B": [45, 1, 200], "C": [97, 33, 64]}
+LENGTHS = {"A": [70, 3, 131], "B": [45, 1, 200], "C": [97, 33, 64], "D": [150, 2, 61]}
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
